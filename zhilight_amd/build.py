@@ -72,12 +72,49 @@ def build(force=False, verbose=False):
         run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs)
     with open(stamp, "w") as fh:
         fh.write(" ".join(flags))
+    build_seq(force, verbose)
     build_hostcpp(force, verbose)
     build_comm(force, verbose)
     build_refcompile(force, verbose)
     build_binding(force, verbose)
     build_refcheck(force, verbose)
     return OUT
+
+
+SEQ_OUT = os.path.join(HERE, "libzhilight_amd_seq.so")
+CSRC_SEQ = os.path.join(HERE, "csrc_seq")
+# hipcc only (its host pass warns that it does not know the feature): no packed fp32 instructions from ordinary float code
+SEQ_FLAGS = FLAGS + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build_seq(force=False, verbose=False):
+    """libzhilight_amd_seq.so: the ragged-batch kernels of the sequence-mixer models (include/zhilight_amd_seq.h; csrc_seq/*.hip).
+    A library of its own: a checkout that serves only such a model compiles these few files and nothing of the quantised decode path."""
+    srcs = sorted(os.path.join(CSRC_SEQ, f) for f in os.listdir(CSRC_SEQ) if f.endswith(".hip"))
+    deps = [os.path.join(CSRC_SEQ, f) for f in os.listdir(CSRC_SEQ) if f.endswith(".h")]
+    deps += [os.path.join(CSRC, "zl_common.h"), os.path.join(HERE, "..", "include", "zhilight_amd.h"),
+             os.path.join(HERE, "..", "include", "zhilight_amd_seq.h")]
+    objdir = os.path.join(HERE, "build", "seq")
+    os.makedirs(objdir, exist_ok=True)
+    objs, jobs = [], []
+    for src in srcs:
+        o = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
+        objs.append(o)
+        if force or _stale(o, [src] + deps):
+            jobs.append([HIPCC] + SEQ_FLAGS + ["-c", src, "-o", o])
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL if not verbose else None, stderr=subprocess.PIPE if not verbose else None)
+
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
+        list(ex.map(run, jobs))
+    if jobs or force or _stale(SEQ_OUT, objs):
+        tmp = SEQ_OUT + ".tmp%d" % os.getpid()
+        run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs)
+        os.replace(tmp, SEQ_OUT)                      # another process that builds at the same time never loads half a file
+    return SEQ_OUT
 
 
 COMM_OUT = os.path.join(HERE, "libzhilight_amd_comm.so")

@@ -1,0 +1,31 @@
+// seq_common.h -- helpers shared by the ragged-batch kernels (gfx950, wave64).
+#pragma once
+#include "../csrc/zl_common.h"
+#include "../../include/zhilight_amd_seq.h"
+
+// element access of the two storage formats: bf16 as raw 16-bit patterns, fp32 as is
+template <int DT> struct SeqT;
+template <> struct SeqT<ZL_BF16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ float ld(const void* p, size_t i) { return ZT<ZL_BF16>::to_f32(reinterpret_cast<const uint16_t*>(p)[i]); }
+    static __device__ __forceinline__ void st(void* p, size_t i, float v) { reinterpret_cast<uint16_t*>(p)[i] = ZT<ZL_BF16>::from_f32(v); }
+};
+template <> struct SeqT<ZL_F32> {
+    typedef float type;
+    static __device__ __forceinline__ float ld(const void* p, size_t i) { return reinterpret_cast<const float*>(p)[i]; }
+    static __device__ __forceinline__ void st(void* p, size_t i, float v) { reinterpret_cast<float*>(p)[i] = v; }
+};
+
+__device__ __forceinline__ float seq_silu(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float seq_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
+__device__ __forceinline__ float seq_softplus(float v) { return v > 20.0f ? v : log1pf(expf(v)); }
+
+static inline bool seq_batch_ok(const zls_batch_t* b) {
+    return b && b->n_seq > 0 && b->n_tok > 0 && b->seq_start && b->seq_pos0 && b->seq_slot && b->tok_seq && b->max_count > 0 &&
+           b->max_count <= b->n_tok;
+}
+
+#define ZLS_DISPATCH(dtype, CALL)                     \
+    if ((dtype) == ZL_BF16) { CALL(ZL_BF16) }         \
+    else if ((dtype) == ZL_F32) { CALL(ZL_F32) }      \
+    else return ZL_EDTYPE;

@@ -1,0 +1,139 @@
+// seq_elem.hip -- the per-token steps between the matrix products of a ragged step: embedding with learned positions, token shift with
+// its carried row, the scalar-gain RMS norm fused with the residual sum, the gathered final norm, PolyNorm.
+// One workgroup per token row; every sum of squares is fp32 (butterfly inside a wave, waves in order).
+#include "seq_common.h"
+
+namespace {
+
+constexpr int kT = 256;
+
+template <int DT>
+__global__ __launch_bounds__(kT) void k_embed(const int32_t* __restrict__ tokens, const void* __restrict__ table, const void* __restrict__ pos_table,
+                                              int vocab, int max_pos, float scale, const zls_batch_t b, float* __restrict__ x, int width) {
+    const int t = blockIdx.x;
+    const int sq = b.tok_seq[t];
+    int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
+    int tok = tokens[t];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    pos = pos >= max_pos ? max_pos - 1 : pos;                       // (the host refuses such a step; never an out-of-bounds read)
+    for (int i = threadIdx.x; i < width; i += kT) {
+        float v = SeqT<DT>::ld(table, (size_t)tok * width + i) * scale;
+        if (pos_table) v += SeqT<DT>::ld(pos_table, (size_t)pos * width + i);
+        x[(size_t)t * width + i] = v;
+    }
+}
+
+// the workgroup of a portion's FIRST token reads prev[slot] and, once it has, replaces it with the portion's last row: no other workgroup
+// touches that slot's row, and each thread reads its own elements before it writes them
+template <int DT>
+__global__ __launch_bounds__(kT) void k_token_shift(const float* __restrict__ x, const float* __restrict__ mix, float* __restrict__ prev,
+                                                    const zls_batch_t b, void* __restrict__ h, int width) {
+    const int t = blockIdx.x;
+    const int sq = b.tok_seq[t];
+    const int first = b.seq_start[sq], last = b.seq_start[sq + 1] - 1;
+    const bool head = t == first;
+    float* pr = prev + (size_t)b.seq_slot[sq] * width;
+    const float* before = head ? pr : x + (size_t)(t - 1) * width;
+    for (int i = threadIdx.x; i < width; i += kT) {
+        const float cur = x[(size_t)t * width + i];
+        const float pv = before[i];
+        SeqT<DT>::st(h, (size_t)t * width + i, cur + (pv - cur) * mix[i]);
+        if (head) pr[i] = x[(size_t)last * width + i];
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kT) void k_add_scalar_norm(float* __restrict__ x, const float* __restrict__ y, float gain, float eps, int width,
+                                                        void* __restrict__ xt) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kT) { const float v = y[row + i]; ss = fmaf(v, v, ss); }
+    ss = zl_block_sum(ss, red);
+    const float f = gain / sqrtf(ss / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += kT) {
+        const float v = x[row + i] + y[row + i] * f;
+        x[row + i] = v;
+        if (xt) SeqT<DT>::st(xt, row + i, v);                   // the sum once more in the serving format, for the next matrix product
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kT) void k_scalar_norm_rows(const float* __restrict__ x, const int32_t* __restrict__ rows, float gain, float eps,
+                                                         int width, void* __restrict__ out) {
+    __shared__ float red[16];
+    const size_t row = (size_t)rows[blockIdx.x] * width, orow = (size_t)blockIdx.x * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kT) { const float v = x[row + i]; ss = fmaf(v, v, ss); }
+    ss = zl_block_sum(ss, red);
+    const float f = gain / sqrtf(ss / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += kT) SeqT<DT>::st(out, orow + i, x[row + i] * f);
+}
+
+template <int DT>
+__global__ __launch_bounds__(kT) void k_polynorm(const float* __restrict__ z, float a, float bq, float c, float e, float eps, int ff,
+                                                 void* __restrict__ out) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * ff;
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int i = threadIdx.x; i < ff; i += kT) {
+        const float v = z[row + i], v2 = v * v, v3 = v2 * v;
+        s1 = fmaf(v, v, s1); s2 = fmaf(v2, v2, s2); s3 = fmaf(v3, v3, s3);
+    }
+    s1 = zl_block_sum(s1, red);
+    s2 = zl_block_sum(s2, red);
+    s3 = zl_block_sum(s3, red);
+    const float f1 = a / sqrtf(s1 / (float)ff + eps), f2 = bq / sqrtf(s2 / (float)ff + eps), f3 = c / sqrtf(s3 / (float)ff + eps);
+    for (int i = threadIdx.x; i < ff; i += kT) {
+        const float v = z[row + i], v2 = v * v;
+        SeqT<DT>::st(out, row + i, v * f1 + v2 * f2 + v2 * v * f3 + e);
+    }
+}
+
+}  // namespace
+
+extern "C" int zls_embed(const int32_t* tokens, const void* table, const void* pos_table, int64_t vocab, int64_t max_positions, float scale,
+                         const zls_batch_t* b, float* x, int64_t width, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(tokens && table && x && seq_batch_ok(b) && width > 0 && vocab > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(!pos_table || max_positions > 0, ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_embed<DT>), dim3(b->n_tok), dim3(kT), 0, (hipStream_t)s, tokens, table, pos_table, (int)vocab, \
+                                    (int)max_positions, scale, *b, x, (int)width);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_token_shift(const float* x, const float* mix, float* prev, const zls_batch_t* b, void* h, int64_t width, int dtype,
+                               zl_stream_t s) {
+    ZL_CHECK_ARG(x && mix && prev && h && seq_batch_ok(b) && width > 0, ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_token_shift<DT>), dim3(b->n_tok), dim3(kT), 0, (hipStream_t)s, x, mix, prev, *b, h, (int)width);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_add_scalar_norm(float* x, const float* y, float gain, float eps, int64_t rows, int64_t width, void* xt, int dtype,
+                                   zl_stream_t s) {
+    ZL_CHECK_ARG(x && y && rows > 0 && width > 0, ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_add_scalar_norm<DT>), dim3((unsigned)rows), dim3(kT), 0, (hipStream_t)s, x, y, gain, eps, (int)width, xt);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_scalar_norm_rows(const float* x, const int32_t* rows, float gain, float eps, int64_t n_rows, int64_t width, void* out,
+                                    int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(x && rows && out && n_rows > 0 && width > 0, ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_scalar_norm_rows<DT>), dim3((unsigned)n_rows), dim3(kT), 0, (hipStream_t)s, x, rows, gain, eps, (int)width, out);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_polynorm(const float* z, const float* coef, float eps, int64_t rows, int64_t ff, void* out, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(z && coef && out && rows > 0 && ff > 0, ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_polynorm<DT>), dim3((unsigned)rows), dim3(kT), 0, (hipStream_t)s, z, coef[0], coef[1], coef[2], coef[3], eps, (int)ff, out);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}

@@ -1,0 +1,225 @@
+// seq_gemm.hip -- y = x . W^T for ANY m, n, k in bf16 or true fp32, fp32 accumulation and (by default) fp32 output.
+//
+// The other dense products of this library (csrc/dense_gemm.hip, dense_gemv.hip) want k % 128 == 0 and 16-bit types; models whose sizes
+// come from a configuration file (widths like 320, projections like 582 columns) and the 32-bit serving mode need a product without
+// shape conditions.  Two kernels:
+//   k_seq_gemv  m <= 8 rows (decode steps): one wave per output column streams its weight row once, 16-byte loads, all rows' sums
+//               in registers, butterfly at the end -- the weight matrix is read exactly once at full width.
+//   k_seq_gemm  more rows (prompt portions, mixed steps): 64 x 64 output tile per workgroup of 4 waves (2 x 2, 32 x 32 each = four
+//               16 x 16 MFMA tiles), 32-k slices of x and W staged through LDS (zero-filled past the edges), the next slice's global
+//               loads issued before the current slice's MFMAs.  bf16: v_mfma_f32_16x16x32_bf16; fp32: v_mfma_f32_16x16x4_f32.
+#include "seq_common.h"
+
+namespace {
+
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBM = 64, kBN = 64, kBK = 32;
+
+struct GemmP {
+    const void* x; const void* w; void* y;
+    int64_t ldx, ldy;
+    int m, n, k, vec;
+};
+
+// ---- tiles in LDS -----------------------------------------------------------------------------------------------------------------
+template <int DT> struct Tile;
+template <> struct Tile<ZL_BF16> {
+    static constexpr int kRow = kBK + 8;                       // 80-byte rows: 16-byte aligned fragments, conflict-free enough
+    typedef uint16_t elem;
+    uint4 r;                                                   // 8 values of one row
+    __device__ __forceinline__ void load(const void* base, int64_t ld, int row, int rows, int k0, int kc, int k, int vec) {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(base) + (size_t)row * ld + k0 + kc;
+        if (row < rows && vec && k0 + kc + 8 <= k) { r = *reinterpret_cast<const uint4*>(p); return; }
+        uint16_t v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (row < rows && k0 + kc + i < k) ? p[i] : (uint16_t)0;
+        r = make_uint4(v[0] | (uint32_t)v[1] << 16, v[2] | (uint32_t)v[3] << 16, v[4] | (uint32_t)v[5] << 16, v[6] | (uint32_t)v[7] << 16);
+    }
+    __device__ __forceinline__ void store(elem* lds, int row, int kc) { *reinterpret_cast<uint4*>(lds + row * kRow + kc) = r; }
+};
+template <> struct Tile<ZL_F32> {
+    static constexpr int kRow = kBK + 4;
+    typedef float elem;
+    float4 r[2];
+    __device__ __forceinline__ void load(const void* base, int64_t ld, int row, int rows, int k0, int kc, int k, int vec) {
+        const float* p = reinterpret_cast<const float*>(base) + (size_t)row * ld + k0 + kc;
+        if (row < rows && vec && k0 + kc + 8 <= k) {
+            r[0] = *reinterpret_cast<const float4*>(p);
+            r[1] = *reinterpret_cast<const float4*>(p + 4);
+            return;
+        }
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (row < rows && k0 + kc + i < k) ? p[i] : 0.f;
+        r[0] = make_float4(v[0], v[1], v[2], v[3]);
+        r[1] = make_float4(v[4], v[5], v[6], v[7]);
+    }
+    __device__ __forceinline__ void store(elem* lds, int row, int kc) {
+        *reinterpret_cast<float4*>(lds + row * kRow + kc) = r[0];
+        *reinterpret_cast<float4*>(lds + row * kRow + kc + 4) = r[1];
+    }
+};
+
+template <int DT, int ODT>
+__global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
+    typedef typename Tile<DT>::elem E;
+    constexpr int RS = Tile<DT>::kRow;
+    __shared__ __attribute__((aligned(16))) E xs[kBM * RS];
+    __shared__ __attribute__((aligned(16))) E ws[kBN * RS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nrow = lane & 15, kq = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
+    const int lrow = tid >> 2, lkc = (tid & 3) * 8;
+
+    f4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
+
+    Tile<DT> tx, tw;
+    tx.load(p.x, p.ldx, m0 + lrow, p.m, 0, lkc, p.k, p.vec);
+    tw.load(p.w, p.k, n0 + lrow, p.n, 0, lkc, p.k, p.vec);
+    for (int k0 = 0; k0 < p.k; k0 += kBK) {
+        __syncthreads();                                        // the previous slice's fragments are consumed
+        tx.store(xs, lrow, lkc);
+        tw.store(ws, lrow, lkc);
+        __syncthreads();
+        if (k0 + kBK < p.k) {                                   // next slice in flight during the MFMAs
+            tx.load(p.x, p.ldx, m0 + lrow, p.m, k0 + kBK, lkc, p.k, p.vec);
+            tw.load(p.w, p.k, n0 + lrow, p.n, k0 + kBK, lkc, p.k, p.vec);
+        }
+        if constexpr (DT == ZL_BF16) {
+            uint4 a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const uint4*>(xs + (wm * 32 + i * 16 + nrow) * RS + 8 * kq);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = *reinterpret_cast<const uint4*>(ws + (wn * 32 + j * 16 + nrow) * RS + 8 * kq);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, a[i]), __builtin_bit_cast(b8, b[j]), acc[i][j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < kBK / 4; ++kk) {
+                float a[2], b[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) a[i] = xs[(wm * 32 + i * 16 + nrow) * RS + 4 * kk + kq];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) b[j] = ws[(wn * 32 + j * 16 + nrow) * RS + 4 * kk + kq];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wn * 32 + j * 16 + nrow;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = m0 + wm * 32 + i * 16 + 4 * kq + r;
+                if (row < p.m && col < p.n) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, acc[i][j][r]);
+            }
+        }
+}
+
+// ---- a few rows: the weights are the traffic -----------------------------------------------------------------------------------------
+template <int DT> struct Vec8;
+template <> struct Vec8<ZL_BF16> {
+    static __device__ __forceinline__ void ld(const void* p, size_t i, float* v) {
+        const uint4 u = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p) + i);
+        const uint32_t q[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = __builtin_bit_cast(float, q[j] << 16);
+            v[2 * j + 1] = __builtin_bit_cast(float, q[j] & 0xffff0000u);
+        }
+    }
+};
+template <> struct Vec8<ZL_F32> {
+    static __device__ __forceinline__ void ld(const void* p, size_t i, float* v) {
+        const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i);
+        const float4 b = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+};
+
+template <int DT, int ODT, int MR>
+__global__ __launch_bounds__(256) void k_seq_gemv(const GemmP p) {
+    const int lane = threadIdx.x & 63;
+    const int col = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (col >= p.n) return;
+    float acc[MR];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) acc[r] = 0.f;
+    const size_t wrow = (size_t)col * p.k;
+    if (p.vec && (p.k & 7) == 0) {
+        for (int k = lane * 8; k < p.k; k += 512) {
+            float wv[8];
+            Vec8<DT>::ld(p.w, wrow + k, wv);
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                if (r < p.m) {
+                    float xv[8];
+                    Vec8<DT>::ld(p.x, (size_t)r * p.ldx + k, xv);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[r] = fmaf(wv[i], xv[i], acc[r]);
+                }
+            }
+        }
+    } else {
+        for (int k = lane; k < p.k; k += 64) {
+            const float wv = SeqT<DT>::ld(p.w, wrow + k);
+#pragma unroll
+            for (int r = 0; r < MR; ++r)
+                if (r < p.m) acc[r] = fmaf(wv, SeqT<DT>::ld(p.x, (size_t)r * p.ldx + k), acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+        const float v = zl_wave_sum(acc[r]);
+        if (lane == 0 && r < p.m) SeqT<ODT>::st(p.y, (size_t)r * p.ldy + col, v);
+    }
+}
+
+template <int DT, int ODT>
+int launch(const GemmP& p, hipStream_t hs) {
+    if (p.m <= 8) {
+        const dim3 grid((unsigned)((p.n + 3) / 4));
+        if (p.m <= 2) hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 2>), grid, dim3(256), 0, hs, p);
+        else if (p.m <= 4) hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 4>), grid, dim3(256), 0, hs, p);
+        else hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 8>), grid, dim3(256), 0, hs, p);
+    } else {
+        const dim3 grid((unsigned)((p.n + kBN - 1) / kBN), (unsigned)((p.m + kBM - 1) / kBM));
+        hipLaunchKernelGGL((k_seq_gemm<DT, ODT>), grid, dim3(256), 0, hs, p);
+    }
+    return zl_launch_status();
+}
+
+}  // namespace
+
+extern "C" int zls_version(void) { return 1; }
+
+extern "C" int zls_gemm_nt(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int64_t m, int64_t n, int64_t k, int dtype,
+                           int out_dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(x && w && y && m > 0 && n > 0 && k > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(ldx >= k && ldy >= n && m < (1 << 30) && n < (1 << 30) && k < (1 << 30), ZL_ESHAPE);
+    ZL_CHECK_ARG((m + kBM - 1) / kBM <= 65535, ZL_ELIMIT);
+    ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
+    ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
+    GemmP p;
+    p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
+    const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
+    p.vec = (k % unit == 0 && ldx % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
+    hipStream_t hs = (hipStream_t)s;
+    if (dtype == ZL_BF16) return out_dtype == ZL_F32 ? launch<ZL_BF16, ZL_F32>(p, hs) : launch<ZL_BF16, ZL_BF16>(p, hs);
+    return launch<ZL_F32, ZL_F32>(p, hs);
+}

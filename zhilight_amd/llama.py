@@ -31,6 +31,7 @@ import torch
 
 from . import ops
 from . import parallel
+from .registry import register_model
 
 
 @dataclass
@@ -799,8 +800,20 @@ class DynBatchContext:
     unquant_kv: Dict[int, torch.Tensor] = field(default_factory=dict)   # INT8 cache: a chunked prompt's temporary fp16 K/V
 
 
+@register_model("llama", "LlamaForCausalLM", "mistral", "MistralForCausalLM", "qwen2", "Qwen2ForCausalLM", "qwen3", "Qwen3ForCausalLM",
+                "cpm_dragonfly", "minicpm", "MiniCPMForCausalLM")
 class LLaMA:
     """model::LLaMA (src/model/llama.cpp:11-165) restricted to the dynamic-batch decode step."""
+    ragged = False                   # driven through its own DynBatchContext (new_context / prefill / step_greedy), not ragged steps
+
+    @classmethod
+    def from_config(cls, cfg: dict, dtype=None, device="cuda:0"):
+        """registry entry: a HF config.json (with its quantization_config, if any) -> an empty model"""
+        qc = cfg.get("quantization_config")
+        return cls(ModelConfig.from_hf(cfg), QuantConfig.from_hf(qc) if qc else QuantConfig(0), device)
+
+    def load_weights(self, ckpt):
+        return self.load_state_dict({k: ckpt[k] for k in ckpt.keys()})
 
     def __init__(self, cfg: ModelConfig, quant: QuantConfig, device="cuda:0", tp=None):
         """tp: parallel.TPGroup (rank, size, process group) for tensor parallelism over the GPUs of a node -- W4 route

@@ -1,0 +1,246 @@
+"""Python face of libzhilight_amd_seq.so (include/zhilight_amd_seq.h): the kernels that run a RAGGED step -- portions of prompts and
+single decoded tokens of several sequences as one flat list of tokens.  As in `ops`: PyTorch supplies device memory and the stream, every
+function enqueues one launcher, and there is no CPU or PyTorch fallback -- without the built library these raise.
+
+The library is built on first use when it is absent (`build.build_seq`: a few files, seconds), so a fresh checkout can serve such a model
+without compiling the quantised decode path.
+"""
+import ctypes as C
+import os
+
+import torch
+
+from ._lib import ZLError
+
+BF16, F32 = 1, 2
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "libzhilight_amd_seq.so")
+SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_add_scalar_norm", "zls_scalar_norm_rows", "zls_polynorm",
+           "zls_latent_store", "zls_latent_attention", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_gated_group_norm"]
+_STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
+           -4: "exceeds a hardware limit"}
+
+
+class Batch(C.Structure):
+    """zls_batch_t"""
+    _fields_ = [("n_seq", C.c_int32), ("n_tok", C.c_int32), ("max_pages", C.c_int32), ("page_size", C.c_int32), ("max_count", C.c_int32),
+                ("reserved", C.c_int32), ("seq_start", C.c_void_p), ("seq_pos0", C.c_void_p), ("seq_slot", C.c_void_p),
+                ("tok_seq", C.c_void_p), ("page_table", C.c_void_p)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(SO_PATH):
+            from . import build
+            build.build_seq()
+        l = C.CDLL(SO_PATH)
+        for name in SYMBOLS:
+            getattr(l, name)
+        _lib = l
+    return _lib
+
+
+def check(status, what):
+    if status != 0:
+        raise ZLError(f"{what}: status {status}: {_STATUS.get(status, 'HIP error')}")
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _i(v):
+    return C.c_int64(int(v))
+
+
+def _f(v):
+    return C.c_float(float(v))
+
+
+def dt_code(dtype):
+    if dtype == torch.bfloat16:
+        return BF16
+    if dtype == torch.float32:
+        return F32
+    raise ZLError(f"the ragged-batch kernels take bfloat16 or float32, not {dtype}")
+
+
+def _cuda(*ts):
+    for t in ts:
+        if t is not None and not (t.is_cuda and t.is_contiguous()):
+            raise ZLError("tensors must be contiguous device tensors")
+
+
+def _f32(*ts):
+    for t in ts:
+        if t is not None and t.dtype != torch.float32:
+            raise ZLError("this argument is fp32 in both modes")
+
+
+class RaggedBatch:
+    """The device-side description of one step (zls_batch_t) and the tensors that own its arrays.
+    seqs: list of (count, pos0, slot, pages) -- pages: the sequence's page ids, enough for pos0 + count tokens."""
+
+    def __init__(self, seqs, page_size, device):
+        n_seq = len(seqs)
+        if n_seq == 0:
+            raise ZLError("an empty step")
+        starts, tok_seq = [0], []
+        max_pages = max(1, max(len(s[3]) for s in seqs))
+        table = []
+        for i, (count, pos0, slot, pages) in enumerate(seqs):
+            if count <= 0 or pos0 < 0 or (pos0 + count + page_size - 1) // page_size > len(pages):
+                raise ZLError("a portion needs count > 0 and pages for all its positions")
+            starts.append(starts[-1] + count)
+            tok_seq += [i] * count
+            table += list(pages) + [0] * (max_pages - len(pages))
+        # ONE host array, one copy: [seq_start | seq_pos0 | seq_slot | tok_seq | page_table]
+        host = torch.tensor(starts + [s[1] for s in seqs] + [s[2] for s in seqs] + tok_seq + table, dtype=torch.int32)
+        self.dev = host.to(device, non_blocking=False)
+        o = [0, n_seq + 1, 2 * n_seq + 1, 3 * n_seq + 1, 3 * n_seq + 1 + starts[-1]]
+        base = self.dev.data_ptr()
+        self.n_seq, self.n_tok, self.starts = n_seq, starts[-1], starts
+        self.counts = [s[0] for s in seqs]
+        self.c = Batch(n_seq, self.n_tok, max_pages, page_size, max(self.counts), 0, *[base + 4 * x for x in o])
+        self.ref = C.byref(self.c)
+
+
+def gemm_nt(x, w, out=None, out_dtype=torch.float32):
+    """x (m, k) . w (n, k)^T -> (m, n); x and w in the serving format, the result fp32 (or that format)."""
+    _cuda(w)
+    if x.dim() != 2 or x.stride(1) != 1 or not x.is_cuda:
+        raise ZLError("gemm_nt: x must be a device matrix with unit column stride")
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or w.dtype != x.dtype:
+        raise ZLError("gemm_nt: size K / dtype mismatch")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    elif out.shape != (m, n) or not out.is_contiguous():
+        raise ZLError("gemm_nt: wrong output")
+    check(lib().zls_gemm_nt(_p(x), _i(x.stride(0)), _p(w), _p(out), _i(n), _i(m), _i(n), _i(k), C.c_int(dt_code(x.dtype)),
+                            C.c_int(dt_code(out.dtype)), _stream()), "gemm_nt")
+    return out
+
+
+def embed(tokens, table, pos_table, scale, batch, out=None):
+    _cuda(tokens, table, pos_table)
+    width = table.shape[1]
+    if out is None:
+        out = torch.empty((batch.n_tok, width), dtype=torch.float32, device=table.device)
+    if tokens.dtype != torch.int32 or tokens.numel() != batch.n_tok:
+        raise ZLError("embed: tokens must be int32, one per flat token")
+    check(lib().zls_embed(_p(tokens), _p(table), _p(pos_table), _i(table.shape[0]), _i(0 if pos_table is None else pos_table.shape[0]),
+                          _f(scale), batch.ref, _p(out), _i(width), C.c_int(dt_code(table.dtype)), _stream()), "embed")
+    return out
+
+
+def token_shift(x, mix, prev, batch, dtype):
+    _cuda(x, mix, prev)
+    _f32(x, mix, prev)
+    width = x.shape[1]
+    if mix.numel() != width or prev.shape[-1] != width:
+        raise ZLError("token_shift: width mismatch")
+    h = torch.empty((batch.n_tok, width), dtype=dtype, device=x.device)
+    check(lib().zls_token_shift(_p(x), _p(mix), _p(prev), batch.ref, _p(h), _i(width), C.c_int(dt_code(dtype)), _stream()), "token_shift")
+    return h
+
+
+def add_scalar_norm(x, y, gain, eps, out_dtype=None):
+    """x += y / rms(y) * gain in place; out_dtype: also return the new x in that format (None: nothing; float32: x itself)"""
+    _cuda(x, y)
+    _f32(x, y)
+    if x.shape != y.shape:
+        raise ZLError("add_scalar_norm: shape mismatch")
+    xt = torch.empty(x.shape, dtype=out_dtype, device=x.device) if out_dtype not in (None, torch.float32) else None
+    check(lib().zls_add_scalar_norm(_p(x), _p(y), _f(gain), _f(eps), _i(x.shape[0]), _i(x.shape[1]), _p(xt),
+                                    C.c_int(BF16 if xt is None else dt_code(out_dtype)), _stream()), "add_scalar_norm")
+    return x if out_dtype == torch.float32 else xt
+
+
+def scalar_norm_rows(x, rows, gain, eps, dtype):
+    _cuda(x, rows)
+    _f32(x)
+    if rows.dtype != torch.int32:
+        raise ZLError("scalar_norm_rows: rows must be int32")
+    out = torch.empty((rows.numel(), x.shape[1]), dtype=dtype, device=x.device)
+    check(lib().zls_scalar_norm_rows(_p(x), _p(rows), _f(gain), _f(eps), _i(rows.numel()), _i(x.shape[1]), _p(out), C.c_int(dt_code(dtype)),
+                                     _stream()), "scalar_norm_rows")
+    return out
+
+
+def polynorm(z, coef, eps, dtype):
+    """coef: four host floats (a, b, c, e)"""
+    _cuda(z)
+    _f32(z)
+    out = torch.empty(z.shape, dtype=dtype, device=z.device)
+    arr = (C.c_float * 4)(*[float(v) for v in coef])
+    check(lib().zls_polynorm(_p(z), arr, _f(eps), _i(z.shape[0]), _i(z.shape[1]), _p(out), C.c_int(dt_code(dtype)), _stream()), "polynorm")
+    return out
+
+
+def latent_store(proj, col0, weight, eps, rank, batch, cache):
+    _cuda(proj, weight, cache)
+    _f32(proj, weight)
+    if cache.dim() != 3 or cache.shape[1] != batch.c.page_size or cache.shape[2] != rank or weight.numel() != rank:
+        raise ZLError("latent_store: cache must be (pages, page_size, rank)")
+    check(lib().zls_latent_store(_p(proj), _i(proj.shape[1]), _i(col0), _p(weight), _f(eps), _i(rank), batch.ref, _p(cache),
+                                 C.c_int(dt_code(cache.dtype)), _stream()), "latent_store")
+
+
+def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim):
+    _cuda(q, gate, w_uk, w_uv, sink, cache)
+    _f32(q, gate, sink)
+    rank = cache.shape[2]
+    if w_uk.shape != (heads * dim, rank) or w_uv.shape != (heads * vdim, rank) or w_uk.dtype != cache.dtype or w_uv.dtype != cache.dtype:
+        raise ZLError("latent_attention: up-projection shapes / dtypes")
+    if sink is not None and sink.numel() != heads:
+        raise ZLError("latent_attention: one sink per head")
+    out = torch.empty((batch.n_tok, heads * vdim), dtype=cache.dtype, device=cache.device)
+    check(lib().zls_latent_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _p(w_uk),
+                                     _p(w_uv), _p(sink), _p(cache), batch.ref, _f(scale), _i(heads), _i(dim), _i(vdim), _i(rank), _p(out),
+                                     C.c_int(dt_code(cache.dtype)), _stream()), "latent_attention")
+    return out
+
+
+def conv_silu(proj, col0, w, bias, tail, batch):
+    """causal convolution + SiLU over `channels` columns of proj from col0, then the carried tail moves on (two launches)"""
+    _cuda(proj, w, bias, tail)
+    _f32(proj, w, bias, tail)
+    channels, taps = w.shape
+    if tail is not None and tuple(tail.shape[1:]) != (taps - 1, channels):
+        raise ZLError("conv_silu: tail must be (slots, taps - 1, channels)")
+    out = torch.empty((batch.n_tok, channels), dtype=torch.float32, device=proj.device)
+    check(lib().zls_conv_silu(_p(proj), _i(proj.shape[1]), _i(col0), _p(w), _p(bias), _p(tail), _i(channels), _i(taps), batch.ref, _p(out),
+                              _stream()), "conv_silu")
+    check(lib().zls_conv_tail_update(_p(proj), _i(proj.shape[1]), _i(col0), _p(tail), _i(channels), _i(taps), batch.ref, _stream()),
+          "conv_tail_update")
+    return out
+
+
+def ssm_scan(xbc, proj, dt_col0, dt_bias, a_log, d, state, heads, vdim, n_state, groups, batch):
+    _cuda(xbc, proj, dt_bias, a_log, d, state)
+    _f32(xbc, proj, dt_bias, a_log, d, state)
+    if xbc.shape[1] != heads * vdim + 2 * groups * n_state or tuple(state.shape[1:]) != (heads, n_state, vdim):
+        raise ZLError("ssm_scan: shapes")
+    y = torch.empty((batch.n_tok, heads * vdim), dtype=torch.float32, device=xbc.device)
+    check(lib().zls_ssm_scan(_p(xbc), _p(proj), _i(proj.shape[1]), _i(dt_col0), _p(dt_bias), _p(a_log), _p(d), _p(state), _i(heads), _i(vdim),
+                             _i(n_state), _i(groups), batch.ref, _p(y), _stream()), "ssm_scan")
+    return y
+
+
+def gated_group_norm(y, proj, z_col0, weight, eps, norm_groups, dtype):
+    _cuda(y, proj, weight)
+    _f32(y, proj, weight)
+    out = torch.empty(y.shape, dtype=dtype, device=y.device)
+    check(lib().zls_gated_group_norm(_p(y), _p(proj), _i(proj.shape[1]), _i(z_col0), _p(weight), _f(eps), _i(y.shape[0]), _i(y.shape[1]),
+                                     _i(norm_groups), _p(out), C.c_int(dt_code(dtype)), _stream()), "gated_group_norm")
+    return out
