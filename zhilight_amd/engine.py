@@ -199,10 +199,10 @@ class Engine:
             p = r.params
             probs = ops.softmax_rows(logits[i:i + 1].contiguous(), temperature=p.temperature)
             k = p.top_k if 0 < p.top_k < probs.shape[1] else probs.shape[1]
-            if k <= 1024:
+            if k <= 64:
                 vals, idx = ops.topk_rows(probs, k)
                 vals, idx = vals[0].double().cpu().numpy(), idx[0].cpu().numpy()
-            else:                                   # (the top-k kernel keeps its candidates in registers / LDS: small k only)
+            else:                                   # (the top-k kernel reads a row once per candidate: small k only)
                 pr = probs[0].double().cpu().numpy()
                 idx = np.argsort(-pr, kind="stable")[:k]
                 vals = pr[idx]
