@@ -434,8 +434,89 @@ def check_logits_against_oracle(model, ctx, dev):
         return {"error": "%s: %s" % (type(e).__name__, str(e)[:300])}
 
 
+SEQ_BENCH_SIZES = {
+    # name: width, attention heads x dim (= value size), latent rank, ff of the two-matrix PolyNorm block, state-space heads x vdim, state,
+    #       groups; the dense Llama-shaped twin has the same width, heads and head size and a gated (three-matrix) ff of 2/3 the size,
+    #       so both carry the same feed-forward parameters
+    "1b": dict(width=2048, heads=16, dim=128, rank=512, ff=8192, m_heads=64, m_vdim=64, state=128, groups=8),
+    "8b": dict(width=4096, heads=32, dim=128, rank=512, ff=14336 * 3 // 2, m_heads=128, m_vdim=64, state=128, groups=8),
+}
+
+
+def bench_sequence_mixers(args, dev):
+    """--mixers: prefill and decode throughput of the ragged-step engine's hybrid model (latent attention + state-space layers, PolyNorm
+    feed-forward; zhilight_amd/tupitar.py) next to the dense bf16 Llama-shaped stack of the same width (zhilight_amd/llama.py, quant type
+    0), random weights, 4 layers each, eager launches on both sides.  One JSON line."""
+    from zhilight_amd.engine import Engine, Entry
+    from zhilight_amd.llama import LLaMA, ModelConfig, QuantConfig
+    from zhilight_amd.tupitar import TupitarConfig, TupitarLayerConfig, TupitarModel
+    seq, vocab, results = args.seq, 32000, []
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    for name in args.mixers.split(","):
+        z = SEQ_BENCH_SIZES[name]
+        att = TupitarLayerConfig("latent_attention", dict(heads=z["heads"], dim=z["dim"], vdim=z["dim"], kv_rank=z["rank"],
+                                                          scale=z["dim"] ** -0.5), dict(ff=z["ff"], kind="dense"))
+        ssm = TupitarLayerConfig("mamba2", dict(heads=z["m_heads"], vdim=z["m_vdim"], state=z["state"], groups=z["groups"], conv=4,
+                                                norm_groups=z["groups"]), dict(ff=z["ff"], kind="dense"))
+        for label, layers in (("latent_attention x4", [att] * 4), ("mamba2 x4", [ssm] * 4), ("hybrid (a, a, m, a)", [att, att, ssm, att])):
+            cfg = TupitarConfig(vocab, z["width"], seq + 64, 1.0, 1e-6, layers)
+            model = TupitarModel(cfg, "bfloat16", dev).init_random(1)
+            toks = torch.randint(0, vocab, (seq,)).tolist()
+            for batch in (1, 8):
+                eng = Engine(model, max_tokens=batch * (seq + 64), max_seqs=batch)
+
+                def prefill():
+                    eng.run_step([Entry("p", toks, [seq - 1])])
+                    eng.release("p")
+                if batch == 1:
+                    ms = timed(prefill, 3)
+                    results.append(dict(model="tupitar " + label, size=name, phase="prefill", tokens=seq, ms=round(ms, 3), tokens_per_s=round(seq / ms * 1e3)))
+                for b in range(batch):
+                    eng.run_step([Entry(f"d{b}", toks[:seq - 40], [])])
+
+                def decode():
+                    eng.run_step([Entry(f"d{b}", [7], [0]) for b in range(batch)])
+                ms = timed(decode, 20)
+                results.append(dict(model="tupitar " + label, size=name, phase="decode", batch=batch, context=seq - 40, ms=round(ms, 3),
+                                    tokens_per_s=round(batch / ms * 1e3)))
+                del eng
+            del model
+        lc = ModelConfig(num_layers=4, dim_model=z["width"], num_heads=z["heads"], dim_head=z["dim"], dim_ff=z["ff"] * 2 // 3 // 128 * 128,
+                         vocab_size=vocab, num_kv_heads=z["heads"], dtype="bfloat16")
+        dense = LLaMA(lc, QuantConfig(0), dev).init_random(1)
+        len_buf = (seq + 64 + 63) // 64 * 64
+        prompt = torch.randint(0, vocab, (seq,), device=dev, dtype=torch.int32)
+        pctx = dense.new_context(1, len_buf, 0)
+        ms = timed(lambda: dense.prefill(pctx, 0, prompt), 3)
+        results.append(dict(model="llama dense", size=name, phase="prefill", tokens=seq, ms=round(ms, 3), tokens_per_s=round(seq / ms * 1e3)))
+        for batch in (1, 8):
+            ctx = dense.new_context(batch, len_buf, seq - 40, fill_random=True)
+            ctx.tokens.copy_(torch.randint(0, vocab, (batch,), device=dev, dtype=torch.int32))
+            ctx.steps_left = 1 << 60                   # the step is repeated in place (no advance): the buffers never fill
+            ms = timed(lambda: dense.encode(ctx), 20)
+            results.append(dict(model="llama dense", size=name, phase="decode", batch=batch, context=seq - 40, ms=round(ms, 3),
+                                tokens_per_s=round(batch / ms * 1e3)))
+        del dense
+    print(json.dumps({"metric": "sequence_mixer_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": 4,
+                      "results": results}))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--mixers", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of the ragged-step engine's latent-attention + "
+                         "state-space model beside the dense Llama-shaped stack of equal width; comma-separated sizes of " + ", ".join(SEQ_BENCH_SIZES))
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
@@ -470,6 +551,8 @@ def main():
         os.environ.setdefault("MASTER_ADDR", "127.0.0.1")
         dist.init_process_group("nccl", rank=rank, world_size=world, device_id=dev)
 
+    if args.mixers:
+        return bench_sequence_mixers(args, dev)
     from zhilight_amd import ops  # noqa: F401  (raises if the HIP library is missing)
     from zhilight_amd.llama import LLaMA, ModelConfig, QuantConfig
 

@@ -42,6 +42,10 @@ int zls_version(void);
  * aligned, element loads otherwise. */
 int zls_gemm_nt(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int64_t m, int64_t n, int64_t k, int dtype, int out_dtype,
                 zl_stream_t s);
+/* The same with gathered rows: row r of x is x[x_rows[r]], row c of w is w[w_rows[c]] (device int32 arrays, NULL: in order; ldw: row
+ * stride of w).  Always the tiled kernel.  The up-projection of cached rows that lie scattered over pages. */
+int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, int64_t ldw, const int32_t* w_rows, void* y,
+                       int64_t ldy, int64_t m, int64_t n, int64_t k, int dtype, int out_dtype, zl_stream_t s);
 
 /* x[t] = table[token[t]] * scale + pos_table[position(t)]  (pos_table NULL: no learned positions).  x fp32 (n_tok, width). */
 int zls_embed(const int32_t* tokens, const void* table, const void* pos_table, int64_t vocab, int64_t max_positions, float scale,
@@ -78,7 +82,17 @@ int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* w
  * w_uk (heads * dim, rank), w_uv (heads * vdim, rank) in `dtype`; out (n_tok, heads * vdim) in `dtype`.  fp32 scores, weights and sums. */
 int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* w_uk,
                          const void* w_uv, const float* sink, const void* cache, const zls_batch_t* b, float scale, int64_t heads,
-                         int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, zl_stream_t s);
+                         int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, zl_stream_t s);
+/* single_only != 0: only sequences that bring ONE token are served (their rows of out written); portions are left to
+ * zls_latent_attention_prompt.
+ *
+ * The same attention for PORTIONS (more than one token) on the matrix cores, bf16 only, over keys and values that the caller has
+ * up-projected for the step: k (n_ctx, ldk >= heads * dim) and vt = V^T (heads * vdim, ldv) in bf16, where sequence i's context rows
+ * 0 .. pos0 + count - 1 stand at rows / columns ctx_start[i] ..; ctx_start[i] is a multiple of 64 (the rows up to the next multiple of 64
+ * exist and hold finite numbers), or -1 for a sequence this call leaves out.  dim, vdim <= 256; ldv % 8 == 0. */
+int zls_latent_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* k,
+                                int64_t ldk, const void* vt, int64_t ldv, const float* sink, const int32_t* ctx_start, const zls_batch_t* b,
+                                float scale, int64_t heads, int64_t dim, int64_t vdim, void* out, int dtype, zl_stream_t s);
 
 /* ---- state-space (Mamba-2) mixer ---------------------------------------------------------------------------------------------- */
 /* Causal per-channel convolution + SiLU over the columns col0 .. col0 + channels - 1 of proj: out[t][c] = silu(bias[c] + sum_k

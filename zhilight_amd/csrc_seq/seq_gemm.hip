@@ -19,8 +19,10 @@ constexpr int kBM = 64, kBN = 64, kBK = 32;
 
 struct GemmP {
     const void* x; const void* w; void* y;
-    int64_t ldx, ldy;
+    int64_t ldx, ldw, ldy;
     int m, n, k, vec;
+    const int32_t* x_rows;                                     // row r of x is x[x_rows[r]] (NULL: r); the same for w
+    const int32_t* w_rows;
 };
 
 // ---- tiles in LDS -----------------------------------------------------------------------------------------------------------------
@@ -81,16 +83,20 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
         for (int j = 0; j < 2; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
     Tile<DT> tx, tw;
-    tx.load(p.x, p.ldx, m0 + lrow, p.m, 0, lkc, p.k, p.vec);
-    tw.load(p.w, p.k, n0 + lrow, p.n, 0, lkc, p.k, p.vec);
+    // a gathered operand: the tile row's source row, looked up once (rows past the edge keep their own, unread, index)
+    const int xr = (p.x_rows && m0 + lrow < p.m) ? p.x_rows[m0 + lrow] : m0 + lrow;
+    const int wr = (p.w_rows && n0 + lrow < p.n) ? p.w_rows[n0 + lrow] : n0 + lrow;
+    const int xlim = m0 + lrow < p.m ? xr + 1 : 0, wlim = n0 + lrow < p.n ? wr + 1 : 0;
+    tx.load(p.x, p.ldx, xr, xlim, 0, lkc, p.k, p.vec);
+    tw.load(p.w, p.ldw, wr, wlim, 0, lkc, p.k, p.vec);
     for (int k0 = 0; k0 < p.k; k0 += kBK) {
         __syncthreads();                                        // the previous slice's fragments are consumed
         tx.store(xs, lrow, lkc);
         tw.store(ws, lrow, lkc);
         __syncthreads();
         if (k0 + kBK < p.k) {                                   // next slice in flight during the MFMAs
-            tx.load(p.x, p.ldx, m0 + lrow, p.m, k0 + kBK, lkc, p.k, p.vec);
-            tw.load(p.w, p.k, n0 + lrow, p.n, k0 + kBK, lkc, p.k, p.vec);
+            tx.load(p.x, p.ldx, xr, xlim, k0 + kBK, lkc, p.k, p.vec);
+            tw.load(p.w, p.ldw, wr, wlim, k0 + kBK, lkc, p.k, p.vec);
         }
         if constexpr (DT == ZL_BF16) {
             uint4 a[2], b[2];
@@ -216,10 +222,36 @@ extern "C" int zls_gemm_nt(const void* x, int64_t ldx, const void* w, void* y, i
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
     GemmP p;
-    p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
+    p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = k; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
+    p.x_rows = p.w_rows = nullptr;
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
     p.vec = (k % unit == 0 && ldx % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
     hipStream_t hs = (hipStream_t)s;
     if (dtype == ZL_BF16) return out_dtype == ZL_F32 ? launch<ZL_BF16, ZL_F32>(p, hs) : launch<ZL_BF16, ZL_BF16>(p, hs);
     return launch<ZL_F32, ZL_F32>(p, hs);
+}
+
+// the same product with GATHERED rows of x and / or w (x_rows / w_rows: device int32 row indices, NULL: the rows in order), always on the
+// tiled matrix-core kernel -- the up-projection of cached rows that lie scattered over pages
+extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, int64_t ldw, const int32_t* w_rows, void* y,
+                                  int64_t ldy, int64_t m, int64_t n, int64_t k, int dtype, int out_dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(x && w && y && m > 0 && n > 0 && k > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(ldx >= k && ldw >= k && ldy >= n && m < (1 << 30) && n < (1 << 30) && k < (1 << 30), ZL_ESHAPE);
+    ZL_CHECK_ARG((m + kBM - 1) / kBM <= 65535, ZL_ELIMIT);
+    ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
+    ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
+    GemmP p;
+    p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
+    p.x_rows = x_rows; p.w_rows = w_rows;
+    const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
+    p.vec = (k % unit == 0 && ldx % unit == 0 && ldw % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
+    const dim3 grid((unsigned)((n + kBN - 1) / kBN), (unsigned)((m + kBM - 1) / kBM));
+    hipStream_t hs = (hipStream_t)s;
+    if (dtype == ZL_BF16) {
+        if (out_dtype == ZL_F32) hipLaunchKernelGGL((k_seq_gemm<ZL_BF16, ZL_F32>), grid, dim3(256), 0, hs, p);
+        else hipLaunchKernelGGL((k_seq_gemm<ZL_BF16, ZL_BF16>), grid, dim3(256), 0, hs, p);
+    } else {
+        hipLaunchKernelGGL((k_seq_gemm<ZL_F32, ZL_F32>), grid, dim3(256), 0, hs, p);
+    }
+    return zl_launch_status();
 }

@@ -42,6 +42,7 @@ class LatentAttention:
         self.name, self.width, self.heads, self.dim, self.vdim, self.rank = name, width, heads, dim, vdim, rank
         self.scale, self.eps, self.has_sink, self.has_gate = float(scale), float(eps), sink, gate
         self.cache = None
+        self.prompt_kernel = True         # bf16 portions on the matrix-core kernel (False: everything on the latent-space kernel)
 
     def load(self, get, prefix, dtype, device):
         H, d, v, r, W = self.heads, self.dim, self.vdim, self.rank, self.width
@@ -76,8 +77,21 @@ class LatentAttention:
         H, d, r = self.heads, self.dim, self.rank
         proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | latent | gate]
         seqops.latent_store(proj, H * d, self.dkv_norm, self.eps, r, batch, self.cache)
-        a = seqops.latent_attention(proj, 0, proj if self.has_gate else None, H * d + r, self.w_uk, self.w_uv, self.sink, self.cache, batch,
-                                    self.scale, H, d, self.vdim)
+        gate = proj if self.has_gate else None
+        prompt = batch.n_ctx > 0 and self.prompt_kernel and h.dtype == torch.bfloat16 and max(d, self.vdim) <= 256
+        a = torch.empty((batch.n_tok, H * self.vdim), dtype=h.dtype, device=h.device)
+        if prompt:
+            # portions: keys and values of their contexts up-projected once (K = C W_uk^T, V^T = W_uv C^T, gathered from the pages), then
+            # the matrix-core kernel; single tokens stay on the latent-space kernel below
+            flat = self.cache.view(-1, r)
+            k = torch.empty((batch.n_ctx, H * d), dtype=h.dtype, device=h.device)
+            vt = torch.empty((H * self.vdim, batch.n_ctx), dtype=h.dtype, device=h.device)
+            seqops.gemm_nt_gather(flat, batch.ctx_rows, self.w_uk, None, batch.n_ctx, H * d, k)
+            seqops.gemm_nt_gather(self.w_uv, None, flat, batch.ctx_rows, H * self.vdim, batch.n_ctx, vt)
+            seqops.latent_attention_prompt(proj, 0, gate, H * d + r, k, vt, self.sink, batch, self.scale, H, d, self.vdim, a)
+        if not prompt or batch.n_single:
+            seqops.latent_attention(proj, 0, gate, H * d + r, self.w_uk, self.w_uv, self.sink, self.cache, batch, self.scale, H, d, self.vdim,
+                                    out=a, single_only=prompt)
         return seqops.gemm_nt(a, self.w_o)
 
 

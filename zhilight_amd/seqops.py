@@ -16,7 +16,7 @@ BF16, F32 = 1, 2
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "libzhilight_amd_seq.so")
 SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_add_scalar_norm", "zls_scalar_norm_rows", "zls_polynorm",
-           "zls_latent_store", "zls_latent_attention", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_gated_group_norm"]
+           "zls_latent_store", "zls_latent_attention", "zls_latent_attention_prompt", "zls_gemm_nt_gather", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_gated_group_norm"]
 _STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
            -4: "exceeds a hardware limit"}
 
@@ -102,13 +102,29 @@ class RaggedBatch:
             starts.append(starts[-1] + count)
             tok_seq += [i] * count
             table += list(pages) + [0] * (max_pages - len(pages))
-        # ONE host array, one copy: [seq_start | seq_pos0 | seq_slot | tok_seq | page_table]
-        host = torch.tensor(starts + [s[1] for s in seqs] + [s[2] for s in seqs] + tok_seq + table, dtype=torch.int32)
+        # the cached rows of every PORTION's whole context, sequence after sequence, each padded to a multiple of 64 rows (the padding
+        # points at the sequence's first row): what the prompt attention's up-projection gathers.  ctx_start: -1 for single tokens
+        ctx_rows, ctx_start = [], []
+        for count, pos0, slot, pages in seqs:
+            if count == 1:
+                ctx_start.append(-1)
+                continue
+            ctx_start.append(len(ctx_rows))
+            n = pos0 + count
+            rows = [pages[j // page_size] * page_size + j % page_size for j in range(n)]
+            ctx_rows += rows + [rows[0]] * (-n % 64)
+        # ONE host array, one copy: [seq_start | seq_pos0 | seq_slot | tok_seq | page_table | ctx_start | ctx_rows]
+        host = torch.tensor(starts + [s[1] for s in seqs] + [s[2] for s in seqs] + tok_seq + table + ctx_start + ctx_rows, dtype=torch.int32)
         self.dev = host.to(device, non_blocking=False)
         o = [0, n_seq + 1, 2 * n_seq + 1, 3 * n_seq + 1, 3 * n_seq + 1 + starts[-1]]
         base = self.dev.data_ptr()
         self.n_seq, self.n_tok, self.starts = n_seq, starts[-1], starts
         self.counts = [s[0] for s in seqs]
+        at = o[4] + len(table)
+        self.ctx_start = self.dev[at:at + n_seq]
+        self.ctx_rows = self.dev[at + n_seq:at + n_seq + len(ctx_rows)]
+        self.n_ctx = len(ctx_rows)
+        self.n_single = sum(1 for c in self.counts if c == 1)
         self.c = Batch(n_seq, self.n_tok, max_pages, page_size, max(self.counts), 0, *[base + 4 * x for x in o])
         self.ref = C.byref(self.c)
 
@@ -196,7 +212,31 @@ def latent_store(proj, col0, weight, eps, rank, batch, cache):
                                  C.c_int(dt_code(cache.dtype)), _stream()), "latent_store")
 
 
-def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim):
+def gemm_nt_gather(x, x_rows, w, w_rows, m, n, out):
+    """rows x_rows of x (all of x: None) times rows w_rows of w, transposed -> out (m, n) in its own dtype"""
+    k = x.shape[-1]
+    if w.shape[-1] != k or x.dtype != w.dtype or out.shape[0] != m or out.shape[1] < n or out.stride(1) != 1:
+        raise ZLError("gemm_nt_gather: shapes")
+    for r in (x_rows, w_rows):
+        if r is not None and (r.dtype != torch.int32 or not r.is_cuda):
+            raise ZLError("gemm_nt_gather: int32 device row indices")
+    check(lib().zls_gemm_nt_gather(_p(x), _i(k), _p(x_rows), _p(w), _i(k), _p(w_rows), _p(out), _i(out.stride(0)), _i(m), _i(n), _i(k),
+                                   C.c_int(dt_code(x.dtype)), C.c_int(dt_code(out.dtype)), _stream()), "gemm_nt_gather")
+    return out
+
+
+def latent_attention_prompt(q, q_col0, gate, g_col0, k, vt, sink, batch, scale, heads, dim, vdim, out):
+    """the portions of the step on the matrix cores; k (n_ctx, heads * dim), vt (heads * vdim, n_ctx) from gemm_nt_gather; writes its rows of out"""
+    _cuda(q, gate, k, vt, sink, out)
+    _f32(q, gate, sink)
+    check(lib().zls_latent_attention_prompt(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0),
+                                            _p(k), _i(k.stride(0)), _p(vt), _i(vt.stride(0)), _p(sink), _p(batch.ctx_start), batch.ref, _f(scale),
+                                            _i(heads), _i(dim), _i(vdim), _p(out), C.c_int(dt_code(out.dtype)), _stream()),
+          "latent_attention_prompt")
+    return out
+
+
+def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim, out=None, single_only=False):
     _cuda(q, gate, w_uk, w_uv, sink, cache)
     _f32(q, gate, sink)
     rank = cache.shape[2]
@@ -204,10 +244,11 @@ def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, sc
         raise ZLError("latent_attention: up-projection shapes / dtypes")
     if sink is not None and sink.numel() != heads:
         raise ZLError("latent_attention: one sink per head")
-    out = torch.empty((batch.n_tok, heads * vdim), dtype=cache.dtype, device=cache.device)
+    if out is None:
+        out = torch.empty((batch.n_tok, heads * vdim), dtype=cache.dtype, device=cache.device)
     check(lib().zls_latent_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _p(w_uk),
                                      _p(w_uv), _p(sink), _p(cache), batch.ref, _f(scale), _i(heads), _i(dim), _i(vdim), _i(rank), _p(out),
-                                     C.c_int(dt_code(cache.dtype)), _stream()), "latent_attention")
+                                     C.c_int(dt_code(cache.dtype)), C.c_int(int(single_only)), _stream()), "latent_attention")
     return out
 
 
