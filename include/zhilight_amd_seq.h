@@ -82,8 +82,11 @@ int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* w
  * w_uk (heads * dim, rank), w_uv (heads * vdim, rank) in `dtype`; out (n_tok, heads * vdim) in `dtype`.  fp32 scores, weights and sums. */
 int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* w_uk,
                          const void* w_uv, const float* sink, const void* cache, const zls_batch_t* b, float scale, int64_t heads,
-                         int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, zl_stream_t s);
-/* single_only != 0: only sequences that bring ONE token are served (their rows of out written); portions are left to
+                         int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, void* workspace, int64_t n_splits,
+                         zl_stream_t s);
+int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t heads, int64_t rank, int64_t n_splits);
+/* The keys of every token are split over n_splits workgroups (the caller picks it so that the launch fills the chip; any value >= 1 is
+ * valid) whose partial results go through `workspace`; rank <= 1024.  single_only != 0: only sequences that bring ONE token are served (their rows of out written); portions are left to
  * zls_latent_attention_prompt.
  *
  * The same attention for PORTIONS (more than one token) on the matrix cores, bf16 only, over keys and values that the caller has
@@ -108,7 +111,7 @@ int zls_conv_tail_update(const float* proj, int64_t ld, int64_t col0, float* tai
  *   dt = softplus(dt_raw + dt_bias_h);  S <- exp(-exp(a_log_h) dt) S + dt B x^T;  y = S^T C + d_h x
  * xbc fp32 (n_tok, heads * vdim + 2 groups * n_state) = [x | B | C] after the convolution; dt_raw = proj[t][dt_col0 + h] (fp32, ld);
  * state fp32 (slots, heads, n_state, vdim), read at the start and written back at the end; y fp32 (n_tok, heads * vdim).
- * Head h uses group h / (heads / groups).  n_state <= 16 * (1024 / vdim) and vdim <= 1024. */
+ * Head h uses group h / (heads / groups).  vdim * ceil_pow2(n_state / 32) <= 1024. */
 int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int64_t dt_col0, const float* dt_bias, const float* a_log, const float* d,
                  float* state, int64_t heads, int64_t vdim, int64_t n_state, int64_t groups, const zls_batch_t* b, float* y, zl_stream_t s);
 

@@ -5,9 +5,10 @@
 // prompts at any offset, and a 32-bit mode.  Only the latent is cached; keys and values are never materialised:
 //     score_j = (W_uk,h^T q_h) . c_j * scale          o_h = W_uv,h . (sum_j w_j c_j)
 // k_latent_store   RMS norm (plain weight) of the down-projection -> the token's cache row
-// k_latent_attn    one wave per (token, head): the query is folded through W_uk once, then 64 keys at a time -- a lane per key for the
-//                  scores (fp32), running maximum / denominator that START at the sink (m = sink, l = 1: the sink counts once, unscaled,
-//                  with no value), a lane per latent column for the weighted sum; W_uv and the gate at the end.
+// k_latent_split   single tokens (and, in 32-bit serving, every token): the query is folded through W_uk, the keys are split over
+//                  workgroups, fp32 VALU; k_latent_combine merges the splits with the sink (it counts once, unscaled, with no value),
+//                  applies W_uv and the gate.
+// k_latent_fa      portions of prompts in bf16 on the matrix cores, over up-projected keys and values.
 #include "seq_common.h"
 
 namespace {
@@ -36,66 +37,145 @@ struct AttnP {
     float scale;
 };
 
-// dynamic LDS: qk[rank] | acc[rank] | prob[64] | rowoff[64] (as int)
+// Split over keys: workgroup = (token, group of 4 heads, split), a wave per head.  A tile of 16 cached rows is staged once in LDS as fp32
+// (row stride rank + 1) and shared by the four heads.  Scores: lane = (key, quarter of the latent columns), two butterflies; weighted sum:
+// a lane owns the latent columns lane, lane + 64, ... (RPL of them, in registers).  Every split leaves (max, denominator, sums) in the
+// workspace; k_latent_combine merges them WITH the sink (m = max(sink, m_i), l = e^(sink - m) + sum l_i e^(m_i - m)), applies W_uv and the
+// gate.  LDS: ct[16][rank + 1] | qk[4][rank]
+// q'_h = scale * W_uk,h^T q_h, once per (token, head): threads along the latent (coalesced rows of W_uk), fp32.  qa (n_tok, heads, rank)
 template <int DT>
-__global__ __launch_bounds__(64) void k_latent_attn(const AttnP p, const zls_batch_t b) {
-    extern __shared__ float lds[];
-    float* qk = lds;
-    float* acc = lds + p.rank;
-    float* prob = acc + p.rank;
-    int* rowoff = reinterpret_cast<int*>(prob + 64);
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(256) void k_latent_absorb(const AttnP p, const zls_batch_t b, float* __restrict__ qa) {
+    const int t = blockIdx.x, h = blockIdx.y;
     const int sq = b.tok_seq[t];
-    if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;     // portions go to the prompt kernel (workgroup-uniform)
+    if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;
+    const float* qh = p.q + (size_t)t * p.ldq + p.q_col0 + (size_t)h * p.dim;
+    for (int r = threadIdx.x; r < p.rank; r += 256) {
+        float a0 = 0.f, a1 = 0.f;
+        int d = 0;
+        for (; d + 1 < p.dim; d += 2) {
+            a0 = fmaf(qh[d], SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d) * p.rank + r), a0);
+            a1 = fmaf(qh[d + 1], SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d + 1) * p.rank + r), a1);
+        }
+        if (d < p.dim) a0 = fmaf(qh[d], SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d) * p.rank + r), a0);
+        qa[((size_t)t * p.heads + h) * p.rank + r] = (a0 + a1) * p.scale;
+    }
+}
+
+template <int DT, int RPL>
+__global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_batch_t b, const float* __restrict__ qa, float* __restrict__ ws,
+                                                      int n_splits) {
+    extern __shared__ float lds[];
+    const int RP = p.rank + 1;
+    float* ct = lds;
+    float* qk = lds + 16 * RP + (threadIdx.x >> 6) * p.rank;
+    const int t = blockIdx.x, split = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = blockIdx.y * 4 + wave;
+    const bool hvalid = h < p.heads;
+    const int sq = b.tok_seq[t];
+    if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;      // portions go to the prompt kernel (workgroup-uniform)
     const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
     const int nkeys = pos + 1;
+    const int chunk = ((nkeys + n_splits - 1) / n_splits + 15) & ~15;
+    const int k0 = split * chunk, k1 = min(nkeys, k0 + chunk);
     const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
-    const float* qh = p.q + (size_t)t * p.ldq + p.q_col0 + (size_t)h * p.dim;
-
-    for (int r = lane; r < p.rank; r += 64) {
-        float a = 0.f;
-        for (int d = 0; d < p.dim; ++d) a = fmaf(qh[d], SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d) * p.rank + r), a);
-        qk[r] = a * p.scale;
-        acc[r] = 0.f;
-    }
-    float m = p.sink ? p.sink[h] : -INFINITY;
-    float l = p.sink ? 1.0f : 0.0f;
-    __syncthreads();
-    for (int j0 = 0; j0 < nkeys; j0 += 64) {
-        const int j = j0 + lane;
-        const bool valid = j < nkeys;
-        float sc = -INFINITY;
-        int row = 0;
-        if (valid) {
-            row = pages[j / b.page_size] * b.page_size + j % b.page_size;
-            const size_t base = (size_t)row * p.rank;
-            float a = 0.f;
-            for (int r = 0; r < p.rank; ++r) a = fmaf(qk[r], SeqT<DT>::ld(p.cache, base + r), a);
-            sc = a;
+    if (hvalid)
+        for (int r = lane; r < p.rank; r += 64) qk[r] = qa[((size_t)t * p.heads + h) * p.rank + r];
+    float acc[RPL];
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) acc[i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+    const int key = lane & 15, quarter = lane >> 4;
+    const int rq = (p.rank + 3) / 4, r_lo = quarter * rq, r_hi = min(p.rank, r_lo + rq);
+    for (int j0 = k0; j0 < k1; j0 += 16) {
+        __syncthreads();
+        {   // 16 threads per key, each walks the row in steps of 16 columns: no division per element, 16 page look-ups per thread
+            const int kk = threadIdx.x >> 4, c0 = threadIdx.x & 15;
+            const int j = j0 + kk;
+            if (j < k1) {
+                const size_t base = ((size_t)pages[j / b.page_size] * b.page_size + j % b.page_size) * p.rank;
+                for (int r = c0; r < p.rank; r += 16) ct[kk * RP + r] = SeqT<DT>::ld(p.cache, base + r);
+            } else {
+                for (int r = c0; r < p.rank; r += 16) ct[kk * RP + r] = 0.f;
+            }
         }
-        const float mnew = fmaxf(m, zl_wave_max(sc));               // finite: key j0 is always valid
-        const float corr = expf(m - mnew);                          // m = -inf (no sink, first tile): 0
+        __syncthreads();
+        if (!hvalid) continue;
+        float sc = 0.f;
+        for (int r = r_lo; r < r_hi; ++r) sc = fmaf(qk[r], ct[key * RP + r], sc);
+        sc += __shfl_xor(sc, 16, 64);
+        sc += __shfl_xor(sc, 32, 64);
+        const bool valid = j0 + key < k1;
+        sc = valid ? sc : -INFINITY;
+        float mx = sc;
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        const float mnew = fmaxf(m, mx);                               // finite: key j0 is valid
+        const float corr = expf(m - mnew);                             // m = -inf at the first tile: 0
         const float pj = valid ? expf(sc - mnew) : 0.f;
-        l = l * corr + zl_wave_sum(pj);
+        float ps = pj;
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) ps += __shfl_xor(ps, off, 64);
+        l = l * corr + ps;
         m = mnew;
-        prob[lane] = pj;
-        rowoff[lane] = row;
-        __syncthreads();
-        const int cnt = min(64, nkeys - j0);
-        for (int r = lane; r < p.rank; r += 64) {
-            float a = acc[r] * corr;
-            for (int jj = 0; jj < cnt; ++jj) a = fmaf(prob[jj], SeqT<DT>::ld(p.cache, (size_t)rowoff[jj] * p.rank + r), a);
-            acc[r] = a;
+        float pk[16];
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) pk[kk] = __shfl(pj, kk, 64);
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) {
+            const int r = lane + 64 * i;
+            if (r < p.rank) {
+                float a = acc[i] * corr;
+#pragma unroll
+                for (int kk = 0; kk < 16; ++kk) a = fmaf(pk[kk], ct[kk * RP + r], a);
+                acc[i] = a;
+            }
         }
-        __syncthreads();
     }
+    if (!hvalid) return;
+    float* out = ws + (((size_t)t * p.heads + h) * n_splits + split) * (p.rank + 2);
+    if (lane == 0) { out[0] = m; out[1] = l; }
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+        const int r = lane + 64 * i;
+        if (r < p.rank) out[2 + r] = acc[i];
+    }
+}
+
+// LDS: acc[rank] | wgt[n_splits]
+template <int DT>
+__global__ __launch_bounds__(256) void k_latent_combine(const AttnP p, const zls_batch_t b, const float* __restrict__ ws, int n_splits) {
+    extern __shared__ float lds[];
+    __shared__ float red[16];
+    float* wgt = lds + p.rank;
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sq = b.tok_seq[t];
+    if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;
+    const float* part = ws + ((size_t)t * p.heads + h) * n_splits * (p.rank + 2);
+    float mloc = p.sink ? p.sink[h] : -INFINITY;                       // threads along the splits: loads in parallel
+    for (int s2 = threadIdx.x; s2 < n_splits; s2 += 256) mloc = fmaxf(mloc, part[(size_t)s2 * (p.rank + 2)]);
+    const float m = zl_block_max(mloc, red);
+    float lloc = 0.f;
+    for (int s2 = threadIdx.x; s2 < n_splits; s2 += 256) {
+        const float ms = part[(size_t)s2 * (p.rank + 2)];
+        const float w = ms == -INFINITY ? 0.f : expf(ms - m);
+        wgt[s2] = w;
+        lloc = fmaf(part[(size_t)s2 * (p.rank + 2) + 1], w, lloc);
+    }
+    const float l = zl_block_sum(lloc, red) + (p.sink ? expf(p.sink[h] - m) : 0.f);      // (its barriers also publish wgt)
+    for (int r = threadIdx.x; r < p.rank; r += 256) {
+        float a = 0.f;
+        for (int s2 = 0; s2 < n_splits; ++s2) a = fmaf(part[(size_t)s2 * (p.rank + 2) + 2 + r], wgt[s2], a);
+        lds[r] = a;
+    }
+    __syncthreads();
     const float g = p.gate ? seq_sigmoid(p.gate[(size_t)t * p.ldg + p.g_col0 + h]) : 1.0f;
     const float inv = g / l;
-    for (int d = lane; d < p.vdim; d += 64) {
+    for (int d = wave; d < p.vdim; d += 4) {                           // a wave per output value, lanes along the latent: coalesced W_uv rows
         const size_t wrow = ((size_t)h * p.vdim + d) * p.rank;
         float a = 0.f;
-        for (int r = 0; r < p.rank; ++r) a = fmaf(SeqT<DT>::ld(p.w_uv, wrow + r), acc[r], a);
-        SeqT<DT>::st(p.out, ((size_t)t * p.heads + h) * p.vdim + d, a * inv);
+        for (int r = lane; r < p.rank; r += 64) a = fmaf(SeqT<DT>::ld(p.w_uv, wrow + r), lds[r], a);
+        a = zl_wave_sum(a);
+        if (lane == 0) SeqT<DT>::st(p.out, ((size_t)t * p.heads + h) * p.vdim + d, a * inv);
     }
 }
 
@@ -259,21 +339,41 @@ extern "C" int zls_latent_store(const float* proj, int64_t ld, int64_t col0, con
     return zl_launch_status();
 }
 
+extern "C" int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t heads, int64_t rank, int64_t n_splits) {
+    if (n_tok <= 0 || heads <= 0 || rank <= 0 || n_splits <= 0) return ZL_EINVAL;
+    return (n_tok * heads * n_splits * (rank + 2) + n_tok * heads * rank) * (int64_t)sizeof(float);    /* partials | folded queries */
+}
+
 extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* w_uk,
                                     const void* w_uv, const float* sink, const void* cache, const zls_batch_t* b, float scale, int64_t heads,
-                                    int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, zl_stream_t s) {
-    ZL_CHECK_ARG(q && w_uk && w_uv && cache && out && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0, ZL_EINVAL);
-    ZL_CHECK_ARG(heads > 0 && dim > 0 && vdim > 0 && rank > 0 && heads <= 65535, ZL_EINVAL);
+                                    int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, void* workspace,
+                                    int64_t n_splits, zl_stream_t s) {
+    ZL_CHECK_ARG(q && w_uk && w_uv && cache && out && workspace && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(heads > 0 && dim > 0 && vdim > 0 && rank > 0 && heads <= 65535 && n_splits > 0 && n_splits <= 65535, ZL_EINVAL);
     ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && (!gate || (g_col0 >= 0 && g_col0 + heads <= ldg)), ZL_ESHAPE);
-    const size_t lds = (2 * (size_t)rank + 128) * sizeof(float);
-    ZL_CHECK_ARG(lds <= 64 * 1024, ZL_ELIMIT);
+    const size_t lds = (16 * ((size_t)rank + 1) + 4 * (size_t)rank) * sizeof(float);
+    ZL_CHECK_ARG(rank <= 1024 && lds <= 64 * 1024, ZL_ELIMIT);
     AttnP p;
     p.q = q; p.gate = gate; p.w_uk = w_uk; p.w_uv = w_uv; p.sink = sink; p.cache = cache; p.out = out;
     p.ldq = ldq; p.ldg = ldg; p.q_col0 = (int)q_col0; p.g_col0 = (int)g_col0;
     p.heads = (int)heads; p.dim = (int)dim; p.vdim = (int)vdim; p.rank = (int)rank; p.scale = scale; p.single_only = single_only;
-#define CALL(DT) hipLaunchKernelGGL((k_latent_attn<DT>), dim3(b->n_tok, (unsigned)heads), dim3(64), lds, (hipStream_t)s, p, *b);
+    const dim3 grid(b->n_tok, (unsigned)((heads + 3) / 4), (unsigned)n_splits);
+    hipStream_t hs = (hipStream_t)s;
+    float* ws = (float*)workspace;
+    float* qa = ws + (size_t)b->n_tok * heads * n_splits * (rank + 2);
+    const int ns = (int)n_splits;
+#define SPLIT(DT, RPL) hipLaunchKernelGGL((k_latent_split<DT, RPL>), grid, dim3(256), lds, hs, p, *b, qa, ws, ns)
+#define CALL(DT)                                  \
+    hipLaunchKernelGGL((k_latent_absorb<DT>), dim3(b->n_tok, (unsigned)heads), dim3(256), 0, hs, p, *b, qa); \
+    if (rank <= 64) SPLIT(DT, 1);                 \
+    else if (rank <= 128) SPLIT(DT, 2);           \
+    else if (rank <= 256) SPLIT(DT, 4);           \
+    else if (rank <= 512) SPLIT(DT, 8);           \
+    else SPLIT(DT, 16);                           \
+    hipLaunchKernelGGL((k_latent_combine<DT>), dim3(b->n_tok, (unsigned)heads), dim3(256), (size_t)(rank + n_splits) * sizeof(float), hs, p, *b, ws, ns);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
+#undef SPLIT
     return zl_launch_status();
 }
 

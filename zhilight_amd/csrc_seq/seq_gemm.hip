@@ -5,8 +5,8 @@
 // shape conditions.  Two kernels:
 //   k_seq_gemv  m <= 8 rows (decode steps): one wave per output column streams its weight row once, 16-byte loads, all rows' sums
 //               in registers, butterfly at the end -- the weight matrix is read exactly once at full width.
-//   k_seq_gemm  more rows (prompt portions, mixed steps): 64 x 64 output tile per workgroup of 4 waves (2 x 2, 32 x 32 each = four
-//               16 x 16 MFMA tiles), 32-k slices of x and W staged through LDS (zero-filled past the edges), the next slice's global
+//   k_seq_gemm  more rows (prompt portions, mixed steps): 128 x 128 or 64 x 64 output tile per workgroup of 4 waves (2 x 2; a wave =
+//               4 x 4 or 2 x 2 MFMA tiles of 16 x 16), 32-k slices of x and W staged through LDS (zero-filled past the edges), the next slice's global
 //               loads issued before the current slice's MFMAs.  bf16: v_mfma_f32_16x16x32_bf16; fp32: v_mfma_f32_16x16x4_f32.
 #include "seq_common.h"
 
@@ -15,7 +15,7 @@ namespace {
 typedef __bf16 b8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
-constexpr int kBM = 64, kBN = 64, kBK = 32;
+constexpr int kBK = 32;
 
 struct GemmP {
     const void* x; const void* w; void* y;
@@ -64,10 +64,12 @@ template <> struct Tile<ZL_F32> {
     }
 };
 
-template <int DT, int ODT>
+// WT x WT MFMA tiles per wave: the workgroup's output tile is (32 WT) x (32 WT)
+template <int DT, int ODT, int WT>
 __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
     typedef typename Tile<DT>::elem E;
     constexpr int RS = Tile<DT>::kRow;
+    constexpr int kBM = 32 * WT, kBN = 32 * WT, PASS = kBM / 64;
     __shared__ __attribute__((aligned(16))) E xs[kBM * RS];
     __shared__ __attribute__((aligned(16))) E ws[kBN * RS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -76,62 +78,74 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
     const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
     const int lrow = tid >> 2, lkc = (tid & 3) * 8;
 
-    f4 acc[2][2];
+    f4 acc[WT][WT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < WT; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
-    Tile<DT> tx, tw;
+    Tile<DT> tx[PASS], tw[PASS];
     // a gathered operand: the tile row's source row, looked up once (rows past the edge keep their own, unread, index)
-    const int xr = (p.x_rows && m0 + lrow < p.m) ? p.x_rows[m0 + lrow] : m0 + lrow;
-    const int wr = (p.w_rows && n0 + lrow < p.n) ? p.w_rows[n0 + lrow] : n0 + lrow;
-    const int xlim = m0 + lrow < p.m ? xr + 1 : 0, wlim = n0 + lrow < p.n ? wr + 1 : 0;
-    tx.load(p.x, p.ldx, xr, xlim, 0, lkc, p.k, p.vec);
-    tw.load(p.w, p.ldw, wr, wlim, 0, lkc, p.k, p.vec);
+    int xr[PASS], wr[PASS], xlim[PASS], wlim[PASS];
+#pragma unroll
+    for (int u = 0; u < PASS; ++u) {
+        const int mr = m0 + lrow + 64 * u, nr = n0 + lrow + 64 * u;
+        xr[u] = (p.x_rows && mr < p.m) ? p.x_rows[mr] : mr;
+        wr[u] = (p.w_rows && nr < p.n) ? p.w_rows[nr] : nr;
+        xlim[u] = mr < p.m ? xr[u] + 1 : 0;
+        wlim[u] = nr < p.n ? wr[u] + 1 : 0;
+        tx[u].load(p.x, p.ldx, xr[u], xlim[u], 0, lkc, p.k, p.vec);
+        tw[u].load(p.w, p.ldw, wr[u], wlim[u], 0, lkc, p.k, p.vec);
+    }
     for (int k0 = 0; k0 < p.k; k0 += kBK) {
         __syncthreads();                                        // the previous slice's fragments are consumed
-        tx.store(xs, lrow, lkc);
-        tw.store(ws, lrow, lkc);
+#pragma unroll
+        for (int u = 0; u < PASS; ++u) {
+            tx[u].store(xs, lrow + 64 * u, lkc);
+            tw[u].store(ws, lrow + 64 * u, lkc);
+        }
         __syncthreads();
         if (k0 + kBK < p.k) {                                   // next slice in flight during the MFMAs
-            tx.load(p.x, p.ldx, xr, xlim, k0 + kBK, lkc, p.k, p.vec);
-            tw.load(p.w, p.ldw, wr, wlim, k0 + kBK, lkc, p.k, p.vec);
+#pragma unroll
+            for (int u = 0; u < PASS; ++u) {
+                tx[u].load(p.x, p.ldx, xr[u], xlim[u], k0 + kBK, lkc, p.k, p.vec);
+                tw[u].load(p.w, p.ldw, wr[u], wlim[u], k0 + kBK, lkc, p.k, p.vec);
+            }
         }
         if constexpr (DT == ZL_BF16) {
-            uint4 a[2], b[2];
+            uint4 a[WT], b[WT];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const uint4*>(xs + (wm * 32 + i * 16 + nrow) * RS + 8 * kq);
+            for (int i = 0; i < WT; ++i) a[i] = *reinterpret_cast<const uint4*>(xs + (wm * 16 * WT + i * 16 + nrow) * RS + 8 * kq);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) b[j] = *reinterpret_cast<const uint4*>(ws + (wn * 32 + j * 16 + nrow) * RS + 8 * kq);
+            for (int j = 0; j < WT; ++j) b[j] = *reinterpret_cast<const uint4*>(ws + (wn * 16 * WT + j * 16 + nrow) * RS + 8 * kq);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < WT; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < WT; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, a[i]), __builtin_bit_cast(b8, b[j]), acc[i][j], 0, 0, 0);
         } else {
 #pragma unroll
             for (int kk = 0; kk < kBK / 4; ++kk) {
-                float a[2], b[2];
+                float a[WT], b[WT];
 #pragma unroll
-                for (int i = 0; i < 2; ++i) a[i] = xs[(wm * 32 + i * 16 + nrow) * RS + 4 * kk + kq];
+                for (int i = 0; i < WT; ++i) a[i] = xs[(wm * 16 * WT + i * 16 + nrow) * RS + 4 * kk + kq];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) b[j] = ws[(wn * 32 + j * 16 + nrow) * RS + 4 * kk + kq];
+                for (int j = 0; j < WT; ++j) b[j] = ws[(wn * 16 * WT + j * 16 + nrow) * RS + 4 * kk + kq];
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < WT; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < WT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
             }
         }
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = n0 + wn * 32 + j * 16 + nrow;
+        for (int j = 0; j < WT; ++j) {
+            const int col = n0 + wn * 16 * WT + j * 16 + nrow;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int row = m0 + wm * 32 + i * 16 + 4 * kq + r;
+                const int row = m0 + wm * 16 * WT + i * 16 + 4 * kq + r;
                 if (row < p.m && col < p.n) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, acc[i][j][r]);
             }
         }
@@ -196,6 +210,19 @@ __global__ __launch_bounds__(256) void k_seq_gemv(const GemmP p) {
     }
 }
 
+// 128 x 128 tiles (four times the MFMAs per LDS fragment) when they still fill the chip, 64 x 64 otherwise
+template <int DT, int ODT>
+void launch_tiled(const GemmP& p, hipStream_t hs) {
+    const int64_t big = (int64_t)((p.m + 127) / 128) * ((p.n + 127) / 128);
+    if (big >= 256) {
+        const dim3 grid((unsigned)((p.n + 127) / 128), (unsigned)((p.m + 127) / 128));
+        hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 4>), grid, dim3(256), 0, hs, p);
+    } else {
+        const dim3 grid((unsigned)((p.n + 63) / 64), (unsigned)((p.m + 63) / 64));
+        hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2>), grid, dim3(256), 0, hs, p);
+    }
+}
+
 template <int DT, int ODT>
 int launch(const GemmP& p, hipStream_t hs) {
     if (p.m <= 8) {
@@ -204,8 +231,7 @@ int launch(const GemmP& p, hipStream_t hs) {
         else if (p.m <= 4) hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 4>), grid, dim3(256), 0, hs, p);
         else hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 8>), grid, dim3(256), 0, hs, p);
     } else {
-        const dim3 grid((unsigned)((p.n + kBN - 1) / kBN), (unsigned)((p.m + kBM - 1) / kBM));
-        hipLaunchKernelGGL((k_seq_gemm<DT, ODT>), grid, dim3(256), 0, hs, p);
+        launch_tiled<DT, ODT>(p, hs);
     }
     return zl_launch_status();
 }
@@ -218,7 +244,7 @@ extern "C" int zls_gemm_nt(const void* x, int64_t ldx, const void* w, void* y, i
                            int out_dtype, zl_stream_t s) {
     ZL_CHECK_ARG(x && w && y && m > 0 && n > 0 && k > 0, ZL_EINVAL);
     ZL_CHECK_ARG(ldx >= k && ldy >= n && m < (1 << 30) && n < (1 << 30) && k < (1 << 30), ZL_ESHAPE);
-    ZL_CHECK_ARG((m + kBM - 1) / kBM <= 65535, ZL_ELIMIT);
+    ZL_CHECK_ARG((m + 63) / 64 <= 65535, ZL_ELIMIT);
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
     GemmP p;
@@ -237,7 +263,7 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
                                   int64_t ldy, int64_t m, int64_t n, int64_t k, int dtype, int out_dtype, zl_stream_t s) {
     ZL_CHECK_ARG(x && w && y && m > 0 && n > 0 && k > 0, ZL_EINVAL);
     ZL_CHECK_ARG(ldx >= k && ldw >= k && ldy >= n && m < (1 << 30) && n < (1 << 30) && k < (1 << 30), ZL_ESHAPE);
-    ZL_CHECK_ARG((m + kBM - 1) / kBM <= 65535, ZL_ELIMIT);
+    ZL_CHECK_ARG((m + 63) / 64 <= 65535, ZL_ELIMIT);
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
     GemmP p;
@@ -245,13 +271,12 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
     p.x_rows = x_rows; p.w_rows = w_rows;
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
     p.vec = (k % unit == 0 && ldx % unit == 0 && ldw % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
-    const dim3 grid((unsigned)((n + kBN - 1) / kBN), (unsigned)((m + kBM - 1) / kBM));
     hipStream_t hs = (hipStream_t)s;
     if (dtype == ZL_BF16) {
-        if (out_dtype == ZL_F32) hipLaunchKernelGGL((k_seq_gemm<ZL_BF16, ZL_F32>), grid, dim3(256), 0, hs, p);
-        else hipLaunchKernelGGL((k_seq_gemm<ZL_BF16, ZL_BF16>), grid, dim3(256), 0, hs, p);
+        if (out_dtype == ZL_F32) launch_tiled<ZL_BF16, ZL_F32>(p, hs);
+        else launch_tiled<ZL_BF16, ZL_BF16>(p, hs);
     } else {
-        hipLaunchKernelGGL((k_seq_gemm<ZL_F32, ZL_F32>), grid, dim3(256), 0, hs, p);
+        launch_tiled<ZL_F32, ZL_F32>(p, hs);
     }
     return zl_launch_status();
 }

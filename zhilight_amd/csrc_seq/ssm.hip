@@ -4,8 +4,8 @@
 // k_conv_silu         a thread per (token, channel); taps before the portion come from the slot's tail (oldest row first)
 // k_conv_tail_update  after it: a thread per (sequence, channel) shifts the tail by the portion's length (rows in increasing order, each
 //                     read before it is overwritten)
-// k_ssm_scan          a workgroup per (sequence, head), vdim x NG threads: thread (p, g) keeps S[n][p] for n = g, g + NG, ... in registers
-//                     (<= 16), walks the portion's tokens in order; y_p is reduced over g through LDS.  dt, the decay and the state are fp32.
+// k_ssm_scan          a workgroup per (sequence, head); the state in registers, tokens staged through LDS 16 at a time and walked in order;
+//                     dt, the decay and the state are fp32.
 // k_gated_group_norm  y * silu(z), then each of the row's equal parts divided by its own root mean square, times the weight
 #include "seq_common.h"
 
@@ -49,58 +49,113 @@ __global__ __launch_bounds__(256) void k_conv_tail_update(const float* __restric
 struct ScanP {
     const float* xbc; const float* proj; const float* dt_bias; const float* a_log; const float* d; float* state; float* y;
     int64_t ld;
-    int dt_col0, heads, vdim, n_state, groups, ng;
+    int dt_col0, heads, vdim, n_state, groups, ngl, npt, kp;
 };
 
-constexpr int kNPT = 16;
+constexpr int kScanSlots = 32;
 
-__global__ __launch_bounds__(1024) void k_ssm_scan(const ScanP p, const zls_batch_t b) {
-    extern __shared__ float red[];                                     // [ng][vdim]
-    const int sq = blockIdx.x, h = blockIdx.y;
-    const int P = p.vdim, N = p.n_state, NG = p.ng;
-    const int pp = threadIdx.x % P, g = threadIdx.x / P;
+// thread = (column p of the head's state, g of ngl adjacent lanes): it keeps S[n][p] for the npt <= NPT states n = g * npt .. in registers.
+// Tokens go through LDS a chunk at a time, one row [x (vdim) | B (n_state) | C (n_state)] each, plus dt and the decay exp(-e^a_log dt).
+// The NEXT chunk's global loads are issued into registers (kScanSlots per thread: slot u = token u / kp, column tid + (u % kp) * threads)
+// before the current chunk is walked, and stored to LDS after it: the walk itself has no barrier and waits for no memory -- y_p needs
+// only a butterfly over the ngl lanes of the column.
+template <int NPT, int MAXT>
+__global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batch_t b) {
+    extern __shared__ float lds[];
+    const int P = p.vdim, N = p.n_state, W = P + 2 * N, KP = p.kp, CH = kScanSlots / KP;
+    // a staged row in LDS: [x, padded to 4 | B: ngl groups of npt (+ 4 unused) | C: the same]: a thread's states are 16-byte aligned runs, the
+    // runs of the ngl lanes of a column start 4 banks apart; everything no token writes (n >= N, the padding) is zero for good
+    const int P4 = (P + 3) & ~3, GS = p.npt + 4, WL = P4 + 2 * p.ngl * GS;
+    float* rows = lds;                             // [CH][WL]
+    float* dts = lds + CH * WL;                    // [CH] dt | [CH] decay
+    for (int i = threadIdx.x; i < CH * WL; i += blockDim.x) rows[i] = 0.f;
+    const int sq = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, nthr = blockDim.x;
+    const int pp = tid / p.ngl, g = tid % p.ngl;
+    const bool active = pp < P;
     const int grp = h / (p.heads / p.groups);
     const int inner = p.heads * P, chan = inner + 2 * p.groups * N;
     const int first = b.seq_start[sq], count = b.seq_start[sq + 1] - first;
     float* st = p.state + ((size_t)b.seq_slot[sq] * p.heads + h) * N * P;
-    float S[kNPT];
+    float S[NPT];
 #pragma unroll
-    for (int i = 0; i < kNPT; ++i) {
-        const int n = g + i * NG;
-        S[i] = n < N ? st[(size_t)n * P + pp] : 0.f;
+    for (int j = 0; j < NPT; ++j) {
+        const int n = g * p.npt + j;
+        S[j] = (active && j < p.npt && n < N) ? st[(size_t)n * P + pp] : 0.f;
     }
     const float rate = expf(p.a_log[h]), bias = p.dt_bias[h], dskip = p.d[h];
-    for (int i = 0; i < count; ++i) {
-        const size_t t = (size_t)(first + i);
-        const float* row = p.xbc + t * chan;
-        const float dt = seq_softplus(p.proj[t * p.ld + p.dt_col0 + h] + bias);
-        const float decay = expf(-rate * dt);
-        const float xv = row[h * P + pp];
-        const float* Bv = row + inner + grp * N;
-        const float* Cv = Bv + p.groups * N;
-        const float dx = dt * xv;
-        float part = 0.f;
+    // where column e of a staged row comes from inside a token's row of xbc
+    auto src_col = [&](int e) { return e < P ? h * P + e : (e < P + N ? inner + grp * N + (e - P) : inner + (p.groups + grp) * N + (e - P - N)); };
+    float pre[kScanSlots], pre_dt = 0.f;
+    auto fetch = [&](int c0) {
+        const int cn = min(CH, count - c0);
 #pragma unroll
-        for (int j = 0; j < kNPT; ++j) {
-            const int n = g + j * NG;
-            if (n < N) {
-                S[j] = fmaf(decay, S[j], Bv[n] * dx);
-                part = fmaf(S[j], Cv[n], part);
+        for (int u = 0; u < kScanSlots; ++u) {
+            const int i = u / KP, e = tid + (u % KP) * nthr;
+            pre[u] = (i < cn && e < W) ? p.xbc[(size_t)(first + c0 + i) * chan + src_col(e)] : 0.f;
+        }
+        if (tid < cn) pre_dt = p.proj[(size_t)(first + c0 + tid) * p.ld + p.dt_col0 + h];
+    };
+    auto publish = [&](int c0) {
+        const int cn = min(CH, count - c0);
+#pragma unroll
+        for (int u = 0; u < kScanSlots; ++u) {
+            const int i = u / KP, e = tid + (u % KP) * nthr;
+            if (i < cn && e < W) {
+                int at = e;
+                if (e >= P) {
+                    const int n = (e - P) % N, half = (e - P) / N;
+                    at = P4 + half * p.ngl * GS + (n / p.npt) * GS + n % p.npt;
+                }
+                rows[i * WL + at] = pre[u];
             }
         }
-        red[g * P + pp] = part;
-        __syncthreads();
-        if (g == 0) {
-            float yv = 0.f;
-            for (int q = 0; q < NG; ++q) yv += red[q * P + pp];
-            p.y[t * inner + h * P + pp] = fmaf(dskip, xv, yv);
+        if (tid < cn) {
+            const float dt = seq_softplus(pre_dt + bias);
+            dts[tid] = dt;
+            dts[CH + tid] = expf(-rate * dt);
         }
+    };
+    fetch(0);
+    for (int c0 = 0; c0 < count; c0 += CH) {
+        const int cn = min(CH, count - c0);
+        __syncthreads();                           // the previous chunk is consumed
+        publish(c0);
         __syncthreads();
-    }
+        if (c0 + CH < count) fetch(c0 + CH);       // in flight during the walk
+        if (active) {
+            for (int i = 0; i < cn; ++i) {
+                const float dt = dts[i], decay = dts[CH + i];
+                const float* row = rows + i * WL;
+                const float xv = row[pp];
+                const float dx = dt * xv;
+                const float4* Bv = reinterpret_cast<const float4*>(row + P4 + g * GS);
+                const float4* Cv = reinterpret_cast<const float4*>(row + P4 + (p.ngl + g) * GS);
+                float part0 = 0.f, part1 = 0.f;
 #pragma unroll
-    for (int i = 0; i < kNPT; ++i) {
-        const int n = g + i * NG;
-        if (n < N) st[(size_t)n * P + pp] = S[i];
+                for (int j = 0; j < NPT; j += 4) {
+                    if (j < p.npt) {                               // (npt is a multiple of 4; states past N see B = C = 0 and stay 0)
+                        const float4 bq = Bv[j >> 2], cq = Cv[j >> 2];
+                        S[j] = fmaf(decay, S[j], bq.x * dx);
+                        S[j + 1] = fmaf(decay, S[j + 1], bq.y * dx);
+                        S[j + 2] = fmaf(decay, S[j + 2], bq.z * dx);
+                        S[j + 3] = fmaf(decay, S[j + 3], bq.w * dx);
+                        part0 = fmaf(S[j], cq.x, part0);
+                        part1 = fmaf(S[j + 1], cq.y, part1);
+                        part0 = fmaf(S[j + 2], cq.z, part0);
+                        part1 = fmaf(S[j + 3], cq.w, part1);
+                    }
+                }
+                float part = part0 + part1;
+                for (int off = 1; off < p.ngl; off <<= 1) part += __shfl_xor(part, off, 64);
+                if (g == 0) p.y[(size_t)(first + c0 + i) * inner + h * P + pp] = fmaf(dskip, xv, part);
+            }
+        }
+    }
+    if (!active) return;
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+        const int n = g * p.npt + j;
+        if (j < p.npt && n < N) st[(size_t)n * P + pp] = S[j];
     }
 }
 
@@ -148,15 +203,30 @@ extern "C" int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int
     ZL_CHECK_ARG(xbc && proj && dt_bias && a_log && d && state && y && seq_batch_ok(b), ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && vdim > 0 && n_state > 0 && groups > 0 && heads % groups == 0 && heads <= 65535, ZL_ESHAPE);
     ZL_CHECK_ARG(dt_col0 >= 0 && dt_col0 + heads <= ld && vdim <= 1024, ZL_ESHAPE);
-    // NG thread rows: enough that a thread keeps at most kNPT state values, and at least 4 waves when the head is small
-    int64_t ng = (n_state + kNPT - 1) / kNPT;
-    while (ng * vdim < 256 && ng < n_state) ++ng;
-    ZL_CHECK_ARG(ng * vdim <= 1024, ZL_ELIMIT);
+    // ngl lanes share a column: the smallest power of two that leaves a thread at most 32 states
+    int64_t ngl = 1;
+    while ((n_state + ngl - 1) / ngl > 32) ngl <<= 1;
+    ZL_CHECK_ARG(ngl <= 64 && ngl * vdim <= 1024, ZL_ELIMIT);
+    const int64_t npt = ((n_state + ngl - 1) / ngl + 3) / 4 * 4;
+    const int64_t threads = (ngl * vdim + 63) / 64 * 64;
     ScanP p;
     p.xbc = xbc; p.proj = proj; p.dt_bias = dt_bias; p.a_log = a_log; p.d = d; p.state = state; p.y = y; p.ld = ld;
-    p.dt_col0 = (int)dt_col0; p.heads = (int)heads; p.vdim = (int)vdim; p.n_state = (int)n_state; p.groups = (int)groups; p.ng = (int)ng;
-    hipLaunchKernelGGL(k_ssm_scan, dim3(b->n_seq, (unsigned)heads), dim3((unsigned)(ng * vdim)), (size_t)(ng * vdim) * sizeof(float),
-                       (hipStream_t)s, p, *b);
+    p.dt_col0 = (int)dt_col0; p.heads = (int)heads; p.vdim = (int)vdim; p.n_state = (int)n_state; p.groups = (int)groups;
+    p.ngl = (int)ngl; p.npt = (int)npt;
+    const int64_t row = vdim + 2 * n_state;
+    const int64_t kp = (row + threads - 1) / threads;                  // register slots a staged token row takes per thread
+    ZL_CHECK_ARG(kp <= kScanSlots, ZL_ELIMIT);
+    p.kp = (int)kp;
+    const size_t lds = (size_t)(kScanSlots / kp) * ((vdim + 3) / 4 * 4 + 2 * ngl * (npt + 4) + 2) * sizeof(float);
+    ZL_CHECK_ARG(lds <= 64 * 1024, ZL_ELIMIT);
+    const dim3 grid(b->n_seq, (unsigned)heads), block((unsigned)threads);
+    hipStream_t hs = (hipStream_t)s;
+    // (up to 256 threads the compiler may use the whole register file for the state and the prefetched chunk)
+#define SCAN(NPT)                                                                                   \
+    if (threads <= 256) hipLaunchKernelGGL((k_ssm_scan<NPT, 256>), grid, block, lds, hs, p, *b);    \
+    else hipLaunchKernelGGL((k_ssm_scan<NPT, 1024>), grid, block, lds, hs, p, *b);
+    if (npt <= 8) { SCAN(8) } else if (npt <= 16) { SCAN(16) } else { SCAN(32) }
+#undef SCAN
     return zl_launch_status();
 }
 

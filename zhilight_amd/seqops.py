@@ -16,7 +16,7 @@ BF16, F32 = 1, 2
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "libzhilight_amd_seq.so")
 SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_add_scalar_norm", "zls_scalar_norm_rows", "zls_polynorm",
-           "zls_latent_store", "zls_latent_attention", "zls_latent_attention_prompt", "zls_gemm_nt_gather", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_gated_group_norm"]
+           "zls_latent_store", "zls_latent_attention", "zls_latent_attention_workspace_bytes", "zls_latent_attention_prompt", "zls_gemm_nt_gather", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_gated_group_norm"]
 _STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
            -4: "exceeds a hardware limit"}
 
@@ -40,6 +40,7 @@ def lib():
         l = C.CDLL(SO_PATH)
         for name in SYMBOLS:
             getattr(l, name)
+        l.zls_latent_attention_workspace_bytes.restype = C.c_int64
         _lib = l
     return _lib
 
@@ -125,6 +126,7 @@ class RaggedBatch:
         self.ctx_rows = self.dev[at + n_seq:at + n_seq + len(ctx_rows)]
         self.n_ctx = len(ctx_rows)
         self.n_single = sum(1 for c in self.counts if c == 1)
+        self.max_ctx = max(s[0] + s[1] for s in seqs)
         self.c = Batch(n_seq, self.n_tok, max_pages, page_size, max(self.counts), 0, *[base + 4 * x for x in o])
         self.ref = C.byref(self.c)
 
@@ -246,9 +248,15 @@ def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, sc
         raise ZLError("latent_attention: one sink per head")
     if out is None:
         out = torch.empty((batch.n_tok, heads * vdim), dtype=cache.dtype, device=cache.device)
+    # enough workgroups to fill the chip (256 CUs, a few per CU), at least 64 keys per split
+    groups = batch.n_tok * ((heads + 3) // 4)
+    n_splits = max(1, min((batch.max_ctx + 63) // 64, (1024 + groups - 1) // groups))
+    ws = torch.empty(int(lib().zls_latent_attention_workspace_bytes(_i(batch.n_tok), _i(heads), _i(rank), _i(n_splits))) // 4,
+                     dtype=torch.float32, device=cache.device)
     check(lib().zls_latent_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _p(w_uk),
                                      _p(w_uv), _p(sink), _p(cache), batch.ref, _f(scale), _i(heads), _i(dim), _i(vdim), _i(rank), _p(out),
-                                     C.c_int(dt_code(cache.dtype)), C.c_int(int(single_only)), _stream()), "latent_attention")
+                                     C.c_int(dt_code(cache.dtype)), C.c_int(int(single_only)), _p(ws), _i(n_splits), _stream()),
+          "latent_attention")
     return out
 
 
