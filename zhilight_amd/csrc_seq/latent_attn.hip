@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void k_latent_store(const float* __restrict__ 
 struct AttnP {
     const float* q; const float* gate; const void* w_uk; const void* w_uv; const float* sink; const void* cache; void* out;
     int64_t ldq, ldg;
-    int q_col0, g_col0, heads, dim, vdim, rank, single_only;
+    int q_col0, g_col0, heads, dim, vdim, rank, single_only, vec;
     float scale;
 };
 
@@ -42,23 +42,36 @@ struct AttnP {
 // a lane owns the latent columns lane, lane + 64, ... (RPL of them, in registers).  Every split leaves (max, denominator, sums) in the
 // workspace; k_latent_combine merges them WITH the sink (m = max(sink, m_i), l = e^(sink - m) + sum l_i e^(m_i - m)), applies W_uv and the
 // gate.  LDS: ct[16][rank + 1] | qk[4][rank]
-// q'_h = scale * W_uk,h^T q_h, once per (token, head): threads along the latent (coalesced rows of W_uk), fp32.  qa (n_tok, heads, rank)
+// q'_h = scale * W_uk,h^T q_h, once per (token, head): workgroup = 64 latent columns (lanes: coalesced rows of W_uk), the four waves
+// take every fourth query dimension, eight loads in flight each; the partial sums meet in LDS.  qa (n_tok, heads, rank) fp32
 template <int DT>
 __global__ __launch_bounds__(256) void k_latent_absorb(const AttnP p, const zls_batch_t b, float* __restrict__ qa) {
-    const int t = blockIdx.x, h = blockIdx.y;
+    __shared__ float part[4][64];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sq = b.tok_seq[t];
     if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;
     const float* qh = p.q + (size_t)t * p.ldq + p.q_col0 + (size_t)h * p.dim;
-    for (int r = threadIdx.x; r < p.rank; r += 256) {
-        float a0 = 0.f, a1 = 0.f;
-        int d = 0;
-        for (; d + 1 < p.dim; d += 2) {
-            a0 = fmaf(qh[d], SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d) * p.rank + r), a0);
-            a1 = fmaf(qh[d + 1], SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d + 1) * p.rank + r), a1);
+    const int r = blockIdx.z * 64 + lane;
+    float acc = 0.f;
+    if (r < p.rank) {
+        for (int d0 = wave; d0 < p.dim; d0 += 32) {
+            float w[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int d = d0 + 4 * u;
+                w[u] = d < p.dim ? SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d) * p.rank + r) : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int d = d0 + 4 * u;
+                acc = fmaf(d < p.dim ? qh[d] : 0.f, w[u], acc);
+            }
         }
-        if (d < p.dim) a0 = fmaf(qh[d], SeqT<DT>::ld(p.w_uk, ((size_t)h * p.dim + d) * p.rank + r), a0);
-        qa[((size_t)t * p.heads + h) * p.rank + r] = (a0 + a1) * p.scale;
     }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && r < p.rank)
+        qa[((size_t)t * p.heads + h) * p.rank + r] = (part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane]) * p.scale;
 }
 
 template <int DT, int RPL>
@@ -93,7 +106,40 @@ __global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_b
             const int j = j0 + kk;
             if (j < k1) {
                 const size_t base = ((size_t)pages[j / b.page_size] * b.page_size + j % b.page_size) * p.rank;
-                for (int r = c0; r < p.rank; r += 16) ct[kk * RP + r] = SeqT<DT>::ld(p.cache, base + r);
+                if (p.vec) {                                           // 16-byte loads, four in flight per thread
+                    constexpr int V = DT == ZL_BF16 ? 8 : 4;
+                    for (int r0 = c0 * V; r0 < p.rank; r0 += 64 * V) {
+                        float v[4][8];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int r = r0 + 16 * V * u;
+                            if (r < p.rank) {
+                                if constexpr (DT == ZL_BF16) {
+                                    const uint4 q4 = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.cache) + base + r);
+                                    const uint32_t w4[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) {
+                                        v[u][2 * e] = __builtin_bit_cast(float, w4[e] << 16);
+                                        v[u][2 * e + 1] = __builtin_bit_cast(float, w4[e] & 0xffff0000u);
+                                    }
+                                } else {
+                                    const float4 q4 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.cache) + base + r);
+                                    v[u][0] = q4.x; v[u][1] = q4.y; v[u][2] = q4.z; v[u][3] = q4.w;
+                                }
+                            }
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int r = r0 + 16 * V * u;
+                            if (r < p.rank) {
+#pragma unroll
+                                for (int e = 0; e < V; ++e) ct[kk * RP + r + e] = v[u][e];
+                            }
+                        }
+                    }
+                } else {
+                    for (int r = c0; r < p.rank; r += 16) ct[kk * RP + r] = SeqT<DT>::ld(p.cache, base + r);
+                }
             } else {
                 for (int r = c0; r < p.rank; r += 16) ct[kk * RP + r] = 0.f;
             }
@@ -170,12 +216,21 @@ __global__ __launch_bounds__(256) void k_latent_combine(const AttnP p, const zls
     __syncthreads();
     const float g = p.gate ? seq_sigmoid(p.gate[(size_t)t * p.ldg + p.g_col0 + h]) : 1.0f;
     const float inv = g / l;
-    for (int d = wave; d < p.vdim; d += 4) {                           // a wave per output value, lanes along the latent: coalesced W_uv rows
-        const size_t wrow = ((size_t)h * p.vdim + d) * p.rank;
-        float a = 0.f;
-        for (int r = lane; r < p.rank; r += 64) a = fmaf(SeqT<DT>::ld(p.w_uv, wrow + r), lds[r], a);
-        a = zl_wave_sum(a);
-        if (lane == 0) SeqT<DT>::st(p.out, ((size_t)t * p.heads + h) * p.vdim + d, a * inv);
+    // a wave per output value, lanes along the latent (coalesced W_uv rows), four values per pass so that their loads are in flight
+    // together; the workgroups of blockIdx.z share the head's outputs
+    for (int d0 = (blockIdx.z * 4 + wave) * 4; d0 < p.vdim; d0 += gridDim.z * 16) {
+        float a[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int r = lane; r < p.rank; r += 64) {
+            const float c = lds[r];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (d0 + u < p.vdim) a[u] = fmaf(SeqT<DT>::ld(p.w_uv, ((size_t)h * p.vdim + d0 + u) * p.rank + r), c, a[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float v = zl_wave_sum(a[u]);
+            if (lane == 0 && d0 + u < p.vdim) SeqT<DT>::st(p.out, ((size_t)t * p.heads + h) * p.vdim + d0 + u, v * inv);
+        }
     }
 }
 
@@ -357,6 +412,7 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
     p.q = q; p.gate = gate; p.w_uk = w_uk; p.w_uv = w_uv; p.sink = sink; p.cache = cache; p.out = out;
     p.ldq = ldq; p.ldg = ldg; p.q_col0 = (int)q_col0; p.g_col0 = (int)g_col0;
     p.heads = (int)heads; p.dim = (int)dim; p.vdim = (int)vdim; p.rank = (int)rank; p.scale = scale; p.single_only = single_only;
+    p.vec = (rank % (dtype == ZL_BF16 ? 8 : 4) == 0 && ((uintptr_t)cache & 15) == 0) ? 1 : 0;
     const dim3 grid(b->n_tok, (unsigned)((heads + 3) / 4), (unsigned)n_splits);
     hipStream_t hs = (hipStream_t)s;
     float* ws = (float*)workspace;
@@ -364,13 +420,13 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
     const int ns = (int)n_splits;
 #define SPLIT(DT, RPL) hipLaunchKernelGGL((k_latent_split<DT, RPL>), grid, dim3(256), lds, hs, p, *b, qa, ws, ns)
 #define CALL(DT)                                  \
-    hipLaunchKernelGGL((k_latent_absorb<DT>), dim3(b->n_tok, (unsigned)heads), dim3(256), 0, hs, p, *b, qa); \
+    hipLaunchKernelGGL((k_latent_absorb<DT>), dim3(b->n_tok, (unsigned)heads, (unsigned)((rank + 63) / 64)), dim3(256), 0, hs, p, *b, qa); \
     if (rank <= 64) SPLIT(DT, 1);                 \
     else if (rank <= 128) SPLIT(DT, 2);           \
     else if (rank <= 256) SPLIT(DT, 4);           \
     else if (rank <= 512) SPLIT(DT, 8);           \
     else SPLIT(DT, 16);                           \
-    hipLaunchKernelGGL((k_latent_combine<DT>), dim3(b->n_tok, (unsigned)heads), dim3(256), (size_t)(rank + n_splits) * sizeof(float), hs, p, *b, ws, ns);
+    hipLaunchKernelGGL((k_latent_combine<DT>), dim3(b->n_tok, (unsigned)heads, (unsigned)((vdim + 31) / 32 > 4 ? 4 : (vdim + 31) / 32)), dim3(256), (size_t)(rank + n_splits) * sizeof(float), hs, p, *b, ws, ns);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
 #undef SPLIT
