@@ -38,10 +38,10 @@ struct AttnP {
 };
 
 // Split over keys: workgroup = (token, group of 4 heads, split), a wave per head.  A tile of 16 cached rows is staged once in LDS as fp32
-// (row stride rank + 1) and shared by the four heads.  Scores: lane = (key, quarter of the latent columns), two butterflies; weighted sum:
+// (row stride rank + 4) and shared by the four heads.  Scores: lane = (key, quarter of the latent columns), two butterflies; weighted sum:
 // a lane owns the latent columns lane, lane + 64, ... (RPL of them, in registers).  Every split leaves (max, denominator, sums) in the
 // workspace; k_latent_combine merges them WITH the sink (m = max(sink, m_i), l = e^(sink - m) + sum l_i e^(m_i - m)), applies W_uv and the
-// gate.  LDS: ct[16][rank + 1] | qk[4][rank]
+// gate.  LDS: ct[16][rank + 4] | qk[4][rank]
 // q'_h = scale * W_uk,h^T q_h, once per (token, head): workgroup = 64 latent columns (lanes: coalesced rows of W_uk), the four waves
 // take every fourth query dimension, eight loads in flight each; the partial sums meet in LDS.  qa (n_tok, heads, rank) fp32
 template <int DT>
@@ -78,7 +78,7 @@ template <int DT, int RPL>
 __global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_batch_t b, const float* __restrict__ qa, float* __restrict__ ws,
                                                       int n_splits) {
     extern __shared__ float lds[];
-    const int RP = p.rank + 1;
+    const int RP = p.rank + 4;                     // rows 16-byte aligned; 4 banks between neighbouring keys
     float* ct = lds;
     float* qk = lds + 16 * RP + (threadIdx.x >> 6) * p.rank;
     const int t = blockIdx.x, split = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -98,7 +98,6 @@ __global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_b
     for (int i = 0; i < RPL; ++i) acc[i] = 0.f;
     float m = -INFINITY, l = 0.f;
     const int key = lane & 15, quarter = lane >> 4;
-    const int rq = (p.rank + 3) / 4, r_lo = quarter * rq, r_hi = min(p.rank, r_lo + rq);
     for (int j0 = k0; j0 < k1; j0 += 16) {
         __syncthreads();
         {   // 16 threads per key, each walks the row in steps of 16 columns: no division per element, 16 page look-ups per thread
@@ -133,7 +132,8 @@ __global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_b
                             const int r = r0 + 16 * V * u;
                             if (r < p.rank) {
 #pragma unroll
-                                for (int e = 0; e < V; ++e) ct[kk * RP + r + e] = v[u][e];
+                                for (int e = 0; e < V; e += 4)
+                                    *reinterpret_cast<float4*>(ct + kk * RP + r + e) = make_float4(v[u][e], v[u][e + 1], v[u][e + 2], v[u][e + 3]);
                             }
                         }
                     }
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_b
         __syncthreads();
         if (!hvalid) continue;
         float sc = 0.f;
-        for (int r = r_lo; r < r_hi; ++r) sc = fmaf(qk[r], ct[key * RP + r], sc);
+        for (int r = quarter; r < p.rank; r += 4) sc = fmaf(qk[r], ct[key * RP + r], sc);    // (key, quarter): 32 banks, two lanes each
         sc += __shfl_xor(sc, 16, 64);
         sc += __shfl_xor(sc, 32, 64);
         const bool valid = j0 + key < k1;
@@ -238,8 +238,9 @@ __global__ __launch_bounds__(256) void k_latent_combine(const AttnP p, const zls
 // Keys and values of a portion's whole context are up-projected once per step into dense K (n_ctx, heads * dim) and V^T (heads * vdim,
 // n_ctx) (zls_gemm_nt_gather over the cached rows; each sequence's rows start at a multiple of 64).  A workgroup = 64 queries of one
 // sequence x one head, a wave = 16 of them.  Per 64-key tile (K and V^T staged in LDS, shared by the four waves):
-//   S^T (16 keys x 16 queries) = K_tile . Q^T on v_mfma_f32_16x16x32_bf16 -- a lane then holds 4 consecutive keys of ONE query, which is
-//   exactly the B operand of v_mfma_f32_16x16x16_bf16, so the weights never travel through LDS:
+//   S^T (16 keys x 16 queries) = K_tile . Q^T on v_mfma_f32_16x16x32_bf16 -- a lane then holds 4 consecutive keys of ONE query; two such
+//   blocks side by side are a B operand of the same instruction with the 32 keys in a permuted order, and V^T is read in that order too,
+//   so the weights never travel through LDS:
 //   O^T (vdim x 16 queries) += V^T_tile . P^T, with P = hi + lo (two bf16 halves: the weights keep 16 bits of mantissa).
 // Scores, running maximum / denominator (starting at the sink: m = sink, l = 1) and the output sums are fp32, per lane = per query.
 typedef __bf16 fa_b8 __attribute__((ext_vector_type(8)));
@@ -339,16 +340,23 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
         const bool dead = mnew == -INFINITY;                                       // nothing seen yet and no sink: keep zeros
         const float corr = dead ? 1.0f : expf(m - mnew);
         float ps = 0.f;
-        fa_s4 hi[4], lo[4];
+        // the 32-key contraction of v_mfma_f32_16x16x32_bf16 may run over the keys in ANY order as long as both operands use the same one:
+        // slot s of lane group kq stands for key 16 (s / 4) + 4 kq + s % 4 of the pair of 16-key blocks, which is how the scores lie here
+        uint32_t hi[2][4], lo[2][4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float pv = (dead || sc[c][r] == -INFINITY) ? 0.f : expf(sc[c][r] - mnew);
-                ps += pv;
-                const uint16_t hb = ZT<ZL_BF16>::from_f32(pv);
-                hi[c][r] = (short)hb;
-                lo[c][r] = (short)ZT<ZL_BF16>::from_f32(pv - ZT<ZL_BF16>::to_f32(hb));
+            for (int r = 0; r < 4; r += 2) {
+                uint16_t hb[2], lb[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float pv = (dead || sc[c][r + e] == -INFINITY) ? 0.f : expf(sc[c][r + e] - mnew);
+                    ps += pv;
+                    hb[e] = ZT<ZL_BF16>::from_f32(pv);
+                    lb[e] = ZT<ZL_BF16>::from_f32(pv - ZT<ZL_BF16>::to_f32(hb[e]));
+                }
+                hi[c >> 1][2 * (c & 1) + (r >> 1)] = hb[0] | (uint32_t)hb[1] << 16;
+                lo[c >> 1][2 * (c & 1) + (r >> 1)] = lb[0] | (uint32_t)lb[1] << 16;
             }
         }
         ps += __shfl_xor(ps, 16, 64);
@@ -359,12 +367,15 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
         for (int dt = 0; dt < DV; ++dt) {
             o[dt] *= corr;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (j0 + 16 * c <= wave_last) {
-                    const uint2 a2 = *reinterpret_cast<const uint2*>(Vs + (16 * dt + nrow) * VR + 16 * c + 4 * kq);
-                    const fa_s4 a = __builtin_bit_cast(fa_s4, a2);
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, hi[c], o[dt], 0, 0, 0);
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, lo[c], o[dt], 0, 0, 0);
+            for (int c2 = 0; c2 < 2; ++c2) {
+                if (j0 + 32 * c2 <= wave_last) {                                    // (a block past the wave's last key has weights 0)
+                    const uint2 a0 = *reinterpret_cast<const uint2*>(Vs + (16 * dt + nrow) * VR + 32 * c2 + 4 * kq);
+                    const uint2 a1 = *reinterpret_cast<const uint2*>(Vs + (16 * dt + nrow) * VR + 32 * c2 + 16 + 4 * kq);
+                    const fa_b8 a = __builtin_bit_cast(fa_b8, make_uint4(a0.x, a0.y, a1.x, a1.y));
+                    const fa_b8 ph = __builtin_bit_cast(fa_b8, make_uint4(hi[c2][0], hi[c2][1], hi[c2][2], hi[c2][3]));
+                    const fa_b8 pl = __builtin_bit_cast(fa_b8, make_uint4(lo[c2][0], lo[c2][1], lo[c2][2], lo[c2][3]));
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ph, o[dt], 0, 0, 0);
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pl, o[dt], 0, 0, 0);
                 }
             }
         }
@@ -406,7 +417,7 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
     ZL_CHECK_ARG(q && w_uk && w_uv && cache && out && workspace && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0, ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && dim > 0 && vdim > 0 && rank > 0 && heads <= 65535 && n_splits > 0 && n_splits <= 65535, ZL_EINVAL);
     ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && (!gate || (g_col0 >= 0 && g_col0 + heads <= ldg)), ZL_ESHAPE);
-    const size_t lds = (16 * ((size_t)rank + 1) + 4 * (size_t)rank) * sizeof(float);
+    const size_t lds = (16 * ((size_t)rank + 4) + 4 * (size_t)rank) * sizeof(float);
     ZL_CHECK_ARG(rank <= 1024 && lds <= 64 * 1024, ZL_ELIMIT);
     AttnP p;
     p.q = q; p.gate = gate; p.w_uk = w_uk; p.w_uv = w_uv; p.sink = sink; p.cache = cache; p.out = out;
