@@ -169,3 +169,16 @@ def test_scheduler_cuts_prompts_and_respects_budgets():
     assert all(sum(e[1] for e in s) <= 100 for s in steps)
     assert {r.rid: len(r.output) for r in eng.finished.values()} == {"r0": 3, "r1": 3, "r2": 3}
     assert not eng.cache.seqs and len(eng.cache.free_pages) == 6
+
+
+def test_seq_header_and_loader_name_the_same_entry_points():
+    import os
+    import re
+    from zhilight_amd import seqops
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "include", "zhilight_amd_seq.h")).read()
+    declared = set(re.findall(r"\b(zls_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(seqops.SYMBOLS)
+    if os.path.exists(seqops.SO_PATH):
+        lib = seqops.lib()
+        assert all(hasattr(lib, n) for n in declared)

@@ -13,8 +13,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libzhilight_amd.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-         "-fno-fast-math", "-ffp-contract=off"]
+BASE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+              "-fno-fast-math", "-ffp-contract=off"]
+# no packed fp32 instructions from ordinary float code (hipcc's host pass warns that it does not know the feature: harmless)
+FLAGS = BASE_FLAGS + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # per-source extras.  w4_slab.hip: its item loops (up to 4 groups x 8 tiles, the next group's normalisation in slices between the
 # items) must unroll completely -- ring slots, accumulators and wait counts are static only then -- and the NORM instantiations
 # exceed the unroller's default budget for `#pragma unroll` (16 K): the ring went to scratch behind dynamic indices
@@ -83,8 +85,7 @@ def build(force=False, verbose=False):
 
 SEQ_OUT = os.path.join(HERE, "libzhilight_amd_seq.so")
 CSRC_SEQ = os.path.join(HERE, "csrc_seq")
-# hipcc only (its host pass warns that it does not know the feature): no packed fp32 instructions from ordinary float code
-SEQ_FLAGS = FLAGS + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+SEQ_FLAGS = FLAGS
 
 
 def build_seq(force=False, verbose=False):
@@ -128,7 +129,8 @@ def build_comm(force=False, verbose=False):
     if not (force or _stale(COMM_OUT, deps)):
         return COMM_OUT
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-shared", "-o", COMM_OUT, src,
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-shared", "-o", COMM_OUT, src,
            "-L" + os.path.join(rocm, "lib"), "-lrccl"]
     if verbose:
         print(" ".join(cmd), flush=True)

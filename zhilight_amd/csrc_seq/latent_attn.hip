@@ -98,53 +98,61 @@ __global__ __launch_bounds__(256) void k_latent_split(const AttnP p, const zls_b
     for (int i = 0; i < RPL; ++i) acc[i] = 0.f;
     float m = -INFINITY, l = 0.f;
     const int key = lane & 15, quarter = lane >> 4;
-    for (int j0 = k0; j0 < k1; j0 += 16) {
-        __syncthreads();
-        {   // 16 threads per key, each walks the row in steps of 16 columns: no division per element, 16 page look-ups per thread
-            const int kk = threadIdx.x >> 4, c0 = threadIdx.x & 15;
-            const int j = j0 + kk;
-            if (j < k1) {
-                const size_t base = ((size_t)pages[j / b.page_size] * b.page_size + j % b.page_size) * p.rank;
-                if (p.vec) {                                           // 16-byte loads, four in flight per thread
-                    constexpr int V = DT == ZL_BF16 ? 8 : 4;
-                    for (int r0 = c0 * V; r0 < p.rank; r0 += 64 * V) {
-                        float v[4][8];
+    // tile fill: 16 threads per key; with aligned rows the NEXT tile's 16-byte loads are issued into registers before the current tile is
+    // worked on and written to LDS after it (8 slots of 16 bytes cover rank <= 1024)
+    constexpr int V = DT == ZL_BF16 ? 8 : 4;
+    const int fk = threadIdx.x >> 4, fc = threadIdx.x & 15;
+    uint4 raw[8];
+    auto row_base = [&](int j) { return ((size_t)pages[j / b.page_size] * b.page_size + j % b.page_size) * p.rank; };
+    auto prefetch = [&](int j0) {
+        const int j = j0 + fk;
+        if (!p.vec || j >= k1) return;
+        const size_t base = row_base(j);
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            const int r = r0 + 16 * V * u;
-                            if (r < p.rank) {
-                                if constexpr (DT == ZL_BF16) {
-                                    const uint4 q4 = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.cache) + base + r);
-                                    const uint32_t w4[4] = {q4.x, q4.y, q4.z, q4.w};
-#pragma unroll
-                                    for (int e = 0; e < 4; ++e) {
-                                        v[u][2 * e] = __builtin_bit_cast(float, w4[e] << 16);
-                                        v[u][2 * e + 1] = __builtin_bit_cast(float, w4[e] & 0xffff0000u);
-                                    }
-                                } else {
-                                    const float4 q4 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.cache) + base + r);
-                                    v[u][0] = q4.x; v[u][1] = q4.y; v[u][2] = q4.z; v[u][3] = q4.w;
-                                }
-                            }
-                        }
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            const int r = r0 + 16 * V * u;
-                            if (r < p.rank) {
-#pragma unroll
-                                for (int e = 0; e < V; e += 4)
-                                    *reinterpret_cast<float4*>(ct + kk * RP + r + e) = make_float4(v[u][e], v[u][e + 1], v[u][e + 2], v[u][e + 3]);
-                            }
-                        }
-                    }
-                } else {
-                    for (int r = c0; r < p.rank; r += 16) ct[kk * RP + r] = SeqT<DT>::ld(p.cache, base + r);
-                }
-            } else {
-                for (int r = c0; r < p.rank; r += 16) ct[kk * RP + r] = 0.f;
+        for (int u = 0; u < 8; ++u) {
+            const int r = (fc + 16 * u) * V;
+            if (r < p.rank) {
+                if constexpr (DT == ZL_BF16) raw[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.cache) + base + r);
+                else raw[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(p.cache) + base + r);
             }
         }
+    };
+    auto publish = [&](int j0) {
+        const int j = j0 + fk;
+        float* dst = ct + fk * RP;
+        if (j >= k1) {
+            for (int r = fc; r < p.rank; r += 16) dst[r] = 0.f;
+        } else if (p.vec) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int r = (fc + 16 * u) * V;
+                if (r < p.rank) {
+                    if constexpr (DT == ZL_BF16) {
+                        const uint32_t w4[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+                        float v[8];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v[2 * e] = __builtin_bit_cast(float, w4[e] << 16);
+                            v[2 * e + 1] = __builtin_bit_cast(float, w4[e] & 0xffff0000u);
+                        }
+                        *reinterpret_cast<float4*>(dst + r) = make_float4(v[0], v[1], v[2], v[3]);
+                        *reinterpret_cast<float4*>(dst + r + 4) = make_float4(v[4], v[5], v[6], v[7]);
+                    } else {
+                        *reinterpret_cast<uint4*>(dst + r) = raw[u];
+                    }
+                }
+            }
+        } else {
+            const size_t base = row_base(j);
+            for (int r = fc; r < p.rank; r += 16) dst[r] = SeqT<DT>::ld(p.cache, base + r);
+        }
+    };
+    prefetch(k0);
+    for (int j0 = k0; j0 < k1; j0 += 16) {
         __syncthreads();
+        publish(j0);
+        __syncthreads();
+        if (j0 + 16 < k1) prefetch(j0 + 16);
         if (!hvalid) continue;
         float sc = 0.f;
         for (int r = quarter; r < p.rank; r += 4) sc = fmaf(qk[r], ct[key * RP + r], sc);    // (key, quarter): 32 banks, two lanes each
@@ -210,6 +218,7 @@ __global__ __launch_bounds__(256) void k_latent_combine(const AttnP p, const zls
     const float l = zl_block_sum(lloc, red) + (p.sink ? expf(p.sink[h] - m) : 0.f);      // (its barriers also publish wgt)
     for (int r = threadIdx.x; r < p.rank; r += 256) {
         float a = 0.f;
+#pragma unroll 8
         for (int s2 = 0; s2 < n_splits; ++s2) a = fmaf(part[(size_t)s2 * (p.rank + 2) + 2 + r], wgt[s2], a);
         lds[r] = a;
     }

@@ -83,32 +83,35 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
         S[j] = (active && j < p.npt && n < N) ? st[(size_t)n * P + pp] : 0.f;
     }
     const float rate = expf(p.a_log[h]), bias = p.dt_bias[h], dskip = p.d[h];
-    // where column e of a staged row comes from inside a token's row of xbc
-    auto src_col = [&](int e) { return e < P ? h * P + e : (e < P + N ? inner + grp * N + (e - P) : inner + (p.groups + grp) * N + (e - P - N)); };
+    // slot u of a thread = (token u / KP of the chunk, column e = tid + (u % KP) * threads of the staged row): where it comes from inside
+    // xbc and where it goes in LDS is the same for every chunk, so both offsets are worked out once (a wave64 VALU instruction costs four
+    // cycles and this loop runs at one wave per SIMD: index arithmetic per chunk would cost more than the recurrence itself)
+    int src_off[kScanSlots], dst_off[kScanSlots];
+#pragma unroll
+    for (int u = 0; u < kScanSlots; ++u) {
+        const int i = u / KP, e = tid + (u % KP) * nthr;
+        int col = h * P + e, at = e;
+        if (e >= P) {
+            const int n = (e - P) % N, half = (e - P) / N;
+            col = inner + (half * p.groups + grp) * N + n;
+            at = P4 + half * p.ngl * GS + (n / p.npt) * GS + n % p.npt;
+        }
+        src_off[u] = e < W ? i * chan + col : -1;
+        dst_off[u] = i * WL + at;
+    }
     float pre[kScanSlots], pre_dt = 0.f;
     auto fetch = [&](int c0) {
         const int cn = min(CH, count - c0);
+        const float* base = p.xbc + (size_t)(first + c0) * chan;
 #pragma unroll
-        for (int u = 0; u < kScanSlots; ++u) {
-            const int i = u / KP, e = tid + (u % KP) * nthr;
-            pre[u] = (i < cn && e < W) ? p.xbc[(size_t)(first + c0 + i) * chan + src_col(e)] : 0.f;
-        }
+        for (int u = 0; u < kScanSlots; ++u) pre[u] = (u < cn * KP && src_off[u] >= 0) ? base[src_off[u]] : 0.f;
         if (tid < cn) pre_dt = p.proj[(size_t)(first + c0 + tid) * p.ld + p.dt_col0 + h];
     };
     auto publish = [&](int c0) {
         const int cn = min(CH, count - c0);
 #pragma unroll
-        for (int u = 0; u < kScanSlots; ++u) {
-            const int i = u / KP, e = tid + (u % KP) * nthr;
-            if (i < cn && e < W) {
-                int at = e;
-                if (e >= P) {
-                    const int n = (e - P) % N, half = (e - P) / N;
-                    at = P4 + half * p.ngl * GS + (n / p.npt) * GS + n % p.npt;
-                }
-                rows[i * WL + at] = pre[u];
-            }
-        }
+        for (int u = 0; u < kScanSlots; ++u)
+            if (u < cn * KP && src_off[u] >= 0) rows[dst_off[u]] = pre[u];
         if (tid < cn) {
             const float dt = seq_softplus(pre_dt + bias);
             dts[tid] = dt;
