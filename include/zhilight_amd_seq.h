@@ -113,7 +113,12 @@ int zls_conv_tail_update(const float* proj, int64_t ld, int64_t col0, float* tai
  * state fp32 (slots, heads, n_state, vdim), read at the start and written back at the end; y fp32 (n_tok, heads * vdim).
  * Head h uses group h / (heads / groups).  vdim * ceil_pow2(n_state / 32) <= 1024. */
 int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int64_t dt_col0, const float* dt_bias, const float* a_log, const float* d,
-                 float* state, int64_t heads, int64_t vdim, int64_t n_state, int64_t groups, const zls_batch_t* b, float* y, zl_stream_t s);
+                 float* state, int64_t heads, int64_t vdim, int64_t n_state, int64_t groups, const zls_batch_t* b, float* y, void* workspace,
+                 int64_t seg_len, zl_stream_t s);
+/* workspace (nullable) and seg_len > 0: portions longer than seg_len tokens run in segments -- all segments from a zero state in parallel,
+ * their start states from a short serial pass, then all segments again from their true start states (the decay is a scalar per head and
+ * token, so a segment acts on its start state as S -> prod(decay) S + S_from_zero).  zls_ssm_scan_workspace_bytes sizes the workspace. */
+int64_t zls_ssm_scan_workspace_bytes(int64_t n_seq, int64_t max_count, int64_t seg_len, int64_t heads, int64_t vdim, int64_t n_state);
 
 /* out = N_g(y * silu(z)) * weight: the gate first, then every one of `norm_groups` equal parts of the row divided by its own root mean
  * square.  y fp32 (rows, inner); z = proj[t][z_col0 ..] fp32; weight fp32 (inner); out in `dtype`. */

@@ -133,7 +133,8 @@ def test_latent_attention_alone(dev, dtype, portions):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("portions", [[90], [1, 1, 2, 3, 40, 1, 42], [2] * 10 + [70]])
 @pytest.mark.parametrize("variant", [0, 1, 2])
-def test_mamba2_alone(dev, dtype, portions, variant):
+@pytest.mark.parametrize("segment", [0, 7, 16])
+def test_mamba2_alone(dev, dtype, portions, variant, segment):
     from zhilight_amd.cache import CacheManager
     from zhilight_amd.mixers import Mamba2Mixer
     cfg = O.small_config(("mamba2",), seed_sizes=variant)
@@ -147,6 +148,7 @@ def test_mamba2_alone(dev, dtype, portions, variant):
     cache = CacheManager(256, 3, dev)
     mix = Mamba2Mixer("m", W, m["heads"], m["vdim"], m["state"], m["groups"], m["conv"], m["norm_groups"], 1e-5).load(lambda n: sub[n], "", dtype, dev)
     mix.bind(cache, dtype)
+    mix.scan_segment = segment                                      # long portions in segments of 7 / 16 tokens (0: one pass)
     cache.admit("other")
     cache.admit("s")                                                # slot 1: slot 0's state stays zero and must stay untouched
     got, at = [], 0
@@ -295,6 +297,9 @@ def test_unequal_batch_equals_each_alone_and_reuses_pages_and_slots(dev, case, d
         alone[k] = run_portions(make(cfg, sd, dtype, dev), k, t, [len(t)])
     assert rel(alone["a"], ref) < tol(dtype)
     eng = make(cfg, sd, dtype, dev, max_tokens=9 * 64, max_seqs=4)  # 12 pages in all; at most 8 at a time
+    for layer in eng.model.layers:                                  # state-space layers: portions above 24 tokens in segments,
+        if hasattr(layer.mixer, "scan_segment"):                    # beside shorter portions and single tokens in the same step
+            layer.mixer.scan_segment = 24
     plan = [
         [("a", 50), ("b", 30), ("c", 2)],
         [("a", 1), ("b", 7), ("c", 100)],                           # b ends here

@@ -50,6 +50,10 @@ struct ScanP {
     const float* xbc; const float* proj; const float* dt_bias; const float* a_log; const float* d; float* state; float* y;
     int64_t ld;
     int dt_col0, heads, vdim, n_state, groups, ngl, npt, kp;
+    // long portions in segments: mode 0 = the whole portion in one workgroup; 1 = a segment from a ZERO state, leaving its end state and the
+    // product of its decays (no y); 2 = a segment from its true start state (seg_init, or the slot's state for segment 0), writing y
+    int mode, seg_len, n_seg;
+    float* seg_state; float* seg_prod; float* seg_init;      // (n_seq, n_seg, heads, n_state, vdim) | (n_seq, n_seg, heads) | like seg_state
 };
 
 constexpr int kScanSlots = 32;
@@ -69,19 +73,26 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
     float* rows = lds;                             // [CH][WL]
     float* dts = lds + CH * WL;                    // [CH] dt | [CH] decay
     for (int i = threadIdx.x; i < CH * WL; i += blockDim.x) rows[i] = 0.f;
-    const int sq = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, nthr = blockDim.x;
+    const int sq = blockIdx.x / p.n_seg, seg = blockIdx.x % p.n_seg, h = blockIdx.y, tid = threadIdx.x, nthr = blockDim.x;
     const int pp = tid / p.ngl, g = tid % p.ngl;
     const bool active = pp < P;
     const int grp = h / (p.heads / p.groups);
     const int inner = p.heads * P, chan = inner + 2 * p.groups * N;
-    const int first = b.seq_start[sq], count = b.seq_start[sq + 1] - first;
+    const int whole = b.seq_start[sq + 1] - b.seq_start[sq];
+    if (seg * p.seg_len >= whole) return;                               // (workgroup-uniform)
+    const int first = b.seq_start[sq] + seg * p.seg_len, count = min(p.seg_len, whole - seg * p.seg_len);
+    const bool last_seg = (seg + 1) * p.seg_len >= whole;
+    if (p.mode == 1 && last_seg) return;                                // nobody starts from the last segment's end state
     float* st = p.state + ((size_t)b.seq_slot[sq] * p.heads + h) * N * P;
+    const size_t seg_at = ((size_t)sq * p.n_seg + seg) * p.heads + h;
+    const float* init = (p.mode == 2 && seg > 0) ? p.seg_init + seg_at * N * P : st;
     float S[NPT];
 #pragma unroll
     for (int j = 0; j < NPT; ++j) {
         const int n = g * p.npt + j;
-        S[j] = (active && j < p.npt && n < N) ? st[(size_t)n * P + pp] : 0.f;
+        S[j] = (p.mode != 1 && active && j < p.npt && n < N) ? init[(size_t)n * P + pp] : 0.f;
     }
+    float prod = 1.0f;
     const float rate = expf(p.a_log[h]), bias = p.dt_bias[h], dskip = p.d[h];
     // slot u of a thread = (token u / KP of the chunk, column e = tid + (u % KP) * threads of the staged row): where it comes from inside
     // xbc and where it goes in LDS is the same for every chunk, so both offsets are worked out once (a wave64 VALU instruction costs four
@@ -128,6 +139,7 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
         if (active) {
             for (int i = 0; i < cn; ++i) {
                 const float dt = dts[i], decay = dts[CH + i];
+                prod *= decay;
                 const float* row = rows + i * WL;
                 const float xv = row[pp];
                 const float dx = dt * xv;
@@ -150,15 +162,36 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
                 }
                 float part = part0 + part1;
                 for (int off = 1; off < p.ngl; off <<= 1) part += __shfl_xor(part, off, 64);
-                if (g == 0) p.y[(size_t)(first + c0 + i) * inner + h * P + pp] = fmaf(dskip, xv, part);
+                if (g == 0 && p.mode != 1) p.y[(size_t)(first + c0 + i) * inner + h * P + pp] = fmaf(dskip, xv, part);
             }
         }
     }
     if (!active) return;
+    if (p.mode == 2 && !last_seg) return;                               // only the portion's last segment leaves the slot's state
+    float* dst = p.mode == 1 ? p.seg_state + seg_at * N * P : st;
 #pragma unroll
     for (int j = 0; j < NPT; ++j) {
         const int n = g * p.npt + j;
-        if (j < p.npt && n < N) st[(size_t)n * P + pp] = S[j];
+        if (j < p.npt && n < N) dst[(size_t)n * P + pp] = S[j];
+    }
+    if (p.mode == 1 && tid == 0) p.seg_prod[seg_at] = prod;
+}
+
+// start states of the segments 1 .. of every long portion: S_{k+1} = (product of segment k's decays) S_k + (segment k's end state from zero),
+// S_0 = the slot's state.  One workgroup per (sequence, head), threads over the state's elements, segments in order.
+__global__ __launch_bounds__(256) void k_ssm_seg_combine(const ScanP p, const zls_batch_t b) {
+    const int sq = blockIdx.x, h = blockIdx.y;
+    const int whole = b.seq_start[sq + 1] - b.seq_start[sq];
+    const int nseg = (whole + p.seg_len - 1) / p.seg_len;
+    const int NPs = p.n_state * p.vdim;
+    const float* st = p.state + ((size_t)b.seq_slot[sq] * p.heads + h) * NPs;
+    for (int e = threadIdx.x; e < NPs; e += 256) {
+        float S = st[e];
+        for (int k = 0; k + 1 < nseg; ++k) {
+            const size_t at = ((size_t)sq * p.n_seg + k) * p.heads + h;
+            S = fmaf(p.seg_prod[at], S, p.seg_state[at * NPs + e]);
+            p.seg_init[(at + p.heads) * NPs + e] = S;                   // segment k + 1 of the same sequence and head
+        }
     }
 }
 
@@ -200,9 +233,15 @@ extern "C" int zls_conv_tail_update(const float* proj, int64_t ld, int64_t col0,
     return zl_launch_status();
 }
 
+extern "C" int64_t zls_ssm_scan_workspace_bytes(int64_t n_seq, int64_t max_count, int64_t seg_len, int64_t heads, int64_t vdim, int64_t n_state) {
+    if (n_seq <= 0 || max_count <= 0 || seg_len <= 0 || heads <= 0 || vdim <= 0 || n_state <= 0) return ZL_EINVAL;
+    const int64_t n_seg = (max_count + seg_len - 1) / seg_len;
+    return n_seq * n_seg * heads * (2 * n_state * vdim + 1) * (int64_t)sizeof(float);
+}
+
 extern "C" int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int64_t dt_col0, const float* dt_bias, const float* a_log,
                             const float* d, float* state, int64_t heads, int64_t vdim, int64_t n_state, int64_t groups, const zls_batch_t* b,
-                            float* y, zl_stream_t s) {
+                            float* y, void* workspace, int64_t seg_len, zl_stream_t s) {
     ZL_CHECK_ARG(xbc && proj && dt_bias && a_log && d && state && y && seq_batch_ok(b), ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && vdim > 0 && n_state > 0 && groups > 0 && heads % groups == 0 && heads <= 65535, ZL_ESHAPE);
     ZL_CHECK_ARG(dt_col0 >= 0 && dt_col0 + heads <= ld && vdim <= 1024, ZL_ESHAPE);
@@ -222,13 +261,36 @@ extern "C" int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int
     p.kp = (int)kp;
     const size_t lds = (size_t)(kScanSlots / kp) * ((vdim + 3) / 4 * 4 + 2 * ngl * (npt + 4) + 2) * sizeof(float);
     ZL_CHECK_ARG(lds <= 64 * 1024, ZL_ELIMIT);
-    const dim3 grid(b->n_seq, (unsigned)heads), block((unsigned)threads);
+    // portions longer than seg_len (with a workspace): every segment from a zero state in parallel, the segments' start states by a short
+    // serial pass over their end states, then every segment again from its true start state -- twice the arithmetic, 1 / segments of the
+    // serial length
+    const bool segmented = workspace && seg_len > 0 && b->max_count > seg_len;
+    const int64_t n_seg = segmented ? (b->max_count + seg_len - 1) / seg_len : 1;
+    p.seg_len = segmented ? (int)seg_len : b->max_count;
+    p.n_seg = (int)n_seg;
+    const int64_t per = (int64_t)b->n_seq * n_seg * heads;
+    p.seg_state = (float*)workspace;
+    p.seg_init = p.seg_state + per * n_state * vdim;
+    p.seg_prod = p.seg_init + per * n_state * vdim;
+    ZL_CHECK_ARG((int64_t)b->n_seq * n_seg <= 0x7fffffff, ZL_ELIMIT);
+    const dim3 grid((unsigned)(b->n_seq * n_seg), (unsigned)heads), block((unsigned)threads);
     hipStream_t hs = (hipStream_t)s;
     // (up to 256 threads the compiler may use the whole register file for the state and the prefetched chunk)
 #define SCAN(NPT)                                                                                   \
     if (threads <= 256) hipLaunchKernelGGL((k_ssm_scan<NPT, 256>), grid, block, lds, hs, p, *b);    \
     else hipLaunchKernelGGL((k_ssm_scan<NPT, 1024>), grid, block, lds, hs, p, *b);
-    if (npt <= 8) { SCAN(8) } else if (npt <= 16) { SCAN(16) } else { SCAN(32) }
+#define SCAN_ANY if (npt <= 8) { SCAN(8) } else if (npt <= 16) { SCAN(16) } else { SCAN(32) }
+    if (!segmented) {
+        p.mode = 0;
+        SCAN_ANY
+    } else {
+        p.mode = 1;
+        SCAN_ANY
+        hipLaunchKernelGGL(k_ssm_seg_combine, dim3(b->n_seq, (unsigned)heads), dim3(256), 0, hs, p, *b);
+        p.mode = 2;
+        SCAN_ANY
+    }
+#undef SCAN_ANY
 #undef SCAN
     return zl_launch_status();
 }

@@ -108,6 +108,7 @@ class Mamba2Mixer:
         self.taps, self.norm_groups, self.eps = taps, norm_groups, float(eps)
         self.inner = heads * vdim
         self.channels = self.inner + 2 * groups * n_state
+        self.scan_segment = None          # tokens per segment of a long portion (None: seqops.SCAN_SEGMENT; 0: never in segments)
 
     def load(self, get, prefix, dtype, device):
         W = self.width
@@ -144,7 +145,7 @@ class Mamba2Mixer:
         proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [z | x | B | C | dt]
         xbc = seqops.conv_silu(proj, self.inner, self.conv_w, self.conv_b, self.tail, batch)
         y = seqops.ssm_scan(xbc, proj, self.inner + self.channels, self.dt_bias, self.a_log, self.d, self.state, self.heads, self.vdim,
-                            self.n_state, self.groups, batch)
+                            self.n_state, self.groups, batch, seg_len=self.scan_segment)
         g = seqops.gated_group_norm(y, proj, 0, self.norm_w, self.eps, self.norm_groups, h.dtype)
         return seqops.gemm_nt(g, self.w_o)
 

@@ -16,7 +16,7 @@ BF16, F32 = 1, 2
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "libzhilight_amd_seq.so")
 SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_add_scalar_norm", "zls_scalar_norm_rows", "zls_polynorm",
-           "zls_latent_store", "zls_latent_attention", "zls_latent_attention_workspace_bytes", "zls_latent_attention_prompt", "zls_gemm_nt_gather", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_gated_group_norm"]
+           "zls_latent_store", "zls_latent_attention", "zls_latent_attention_workspace_bytes", "zls_latent_attention_prompt", "zls_gemm_nt_gather", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_ssm_scan_workspace_bytes", "zls_gated_group_norm"]
 _STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
            -4: "exceeds a hardware limit"}
 
@@ -41,6 +41,7 @@ def lib():
         for name in SYMBOLS:
             getattr(l, name)
         l.zls_latent_attention_workspace_bytes.restype = C.c_int64
+        l.zls_ssm_scan_workspace_bytes.restype = C.c_int64
         _lib = l
     return _lib
 
@@ -275,14 +276,22 @@ def conv_silu(proj, col0, w, bias, tail, batch):
     return out
 
 
-def ssm_scan(xbc, proj, dt_col0, dt_bias, a_log, d, state, heads, vdim, n_state, groups, batch):
+SCAN_SEGMENT = 256      # tokens per segment of a long portion (ssm_scan)
+
+
+def ssm_scan(xbc, proj, dt_col0, dt_bias, a_log, d, state, heads, vdim, n_state, groups, batch, seg_len=None):
     _cuda(xbc, proj, dt_bias, a_log, d, state)
     _f32(xbc, proj, dt_bias, a_log, d, state)
     if xbc.shape[1] != heads * vdim + 2 * groups * n_state or tuple(state.shape[1:]) != (heads, n_state, vdim):
         raise ZLError("ssm_scan: shapes")
     y = torch.empty((batch.n_tok, heads * vdim), dtype=torch.float32, device=xbc.device)
+    seg_len = SCAN_SEGMENT if seg_len is None else seg_len
+    ws = None
+    if seg_len > 0 and batch.c.max_count > seg_len:
+        ws = torch.empty(int(lib().zls_ssm_scan_workspace_bytes(_i(batch.n_seq), _i(batch.c.max_count), _i(seg_len), _i(heads), _i(vdim),
+                                                                _i(n_state))) // 4, dtype=torch.float32, device=xbc.device)
     check(lib().zls_ssm_scan(_p(xbc), _p(proj), _i(proj.shape[1]), _i(dt_col0), _p(dt_bias), _p(a_log), _p(d), _p(state), _i(heads), _i(vdim),
-                             _i(n_state), _i(groups), batch.ref, _p(y), _stream()), "ssm_scan")
+                             _i(n_state), _i(groups), batch.ref, _p(y), _p(ws), _i(seg_len), _stream()), "ssm_scan")
     return y
 
 
