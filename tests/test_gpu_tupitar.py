@@ -52,7 +52,8 @@ def tokens_of(cfg, n, seed):
 # mechanisms alone
 # ------------------------------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("m,n,k", [(1, 70, 96), (3, 129, 100), (8, 64, 90), (9, 200, 96), (70, 65, 33), (130, 582, 320), (257, 48, 1024)])
+@pytest.mark.parametrize("m,n,k", [(1, 70, 96), (3, 129, 100), (8, 64, 90), (9, 200, 96), (5, 70, 96), (16, 33, 320), (12, 129, 1000), (4, 17, 8),
+                                   (70, 65, 33), (130, 582, 320), (257, 48, 1024), (300, 260, 264)])
 def test_gemm_any_shape(dev, dtype, m, n, k):
     from zhilight_amd import seqops
     g = torch.Generator().manual_seed(m * 1000 + n + k)

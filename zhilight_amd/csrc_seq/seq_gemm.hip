@@ -3,8 +3,9 @@
 // The other dense products of this library (csrc/dense_gemm.hip, dense_gemv.hip) want k % 128 == 0 and 16-bit types; models whose sizes
 // come from a configuration file (widths like 320, projections like 582 columns) and the 32-bit serving mode need a product without
 // shape conditions.  Two kernels:
-//   k_seq_gemv  m <= 8 rows (decode steps): one wave per output column streams its weight row once, 16-byte loads, all rows' sums
-//               in registers, butterfly at the end -- the weight matrix is read exactly once at full width.
+//   k_seq_gemv  m <= 8 rows (decode steps): a wave streams the weight rows of 1 / 2 / 4 output columns (for <= 2 / 4 / 8 activation rows)
+//               once, 16-byte loads, all sums in registers, butterflies at the end -- the weight matrix is read exactly once.
+//   k_seq_gemv_mfma  3 .. 16 rows in bf16: the same streaming with the products on the matrix cores (see there).
 //   k_seq_gemm  more rows (prompt portions, mixed steps): 128 x 128 or 64 x 64 output tile per workgroup of 4 waves (2 x 2; a wave =
 //               4 x 4 or 2 x 2 MFMA tiles of 16 x 16), 32-k slices of x and W staged through LDS (zero-filled past the edges), the next slice's global
 //               loads issued before the current slice's MFMAs.  bf16: v_mfma_f32_16x16x32_bf16; fp32: v_mfma_f32_16x16x4_f32.
@@ -172,42 +173,96 @@ template <> struct Vec8<ZL_F32> {
     }
 };
 
-template <int DT, int ODT, int MR>
+// CPW output columns per wave: the activation rows (L2) are read once per CPW weight rows (HBM) -- with 8 rows and one column per wave
+// the activations would be eight times the weight traffic
+template <int DT, int ODT, int MR, int CPW>
 __global__ __launch_bounds__(256) void k_seq_gemv(const GemmP p) {
     const int lane = threadIdx.x & 63;
-    const int col = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (col >= p.n) return;
-    float acc[MR];
+    const int col0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * CPW;
+    if (col0 >= p.n) return;
+    float acc[MR][CPW];
 #pragma unroll
-    for (int r = 0; r < MR; ++r) acc[r] = 0.f;
-    const size_t wrow = (size_t)col * p.k;
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) acc[r][c] = 0.f;
+    size_t wrow[CPW];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) wrow[c] = (size_t)min(col0 + c, p.n - 1) * p.k;      // (a column past the edge: the last one, never stored)
     if (p.vec && (p.k & 7) == 0) {
         for (int k = lane * 8; k < p.k; k += 512) {
-            float wv[8];
-            Vec8<DT>::ld(p.w, wrow + k, wv);
+            float wv[CPW][8];
+#pragma unroll
+            for (int c = 0; c < CPW; ++c) Vec8<DT>::ld(p.w, wrow[c] + k, wv[c]);
 #pragma unroll
             for (int r = 0; r < MR; ++r) {
                 if (r < p.m) {
                     float xv[8];
                     Vec8<DT>::ld(p.x, (size_t)r * p.ldx + k, xv);
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) acc[r] = fmaf(wv[i], xv[i], acc[r]);
+                    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) acc[r][c] = fmaf(wv[c][i], xv[i], acc[r][c]);
                 }
             }
         }
     } else {
         for (int k = lane; k < p.k; k += 64) {
-            const float wv = SeqT<DT>::ld(p.w, wrow + k);
+            float wv[CPW];
+#pragma unroll
+            for (int c = 0; c < CPW; ++c) wv[c] = SeqT<DT>::ld(p.w, wrow[c] + k);
 #pragma unroll
             for (int r = 0; r < MR; ++r)
-                if (r < p.m) acc[r] = fmaf(wv, SeqT<DT>::ld(p.x, (size_t)r * p.ldx + k), acc[r]);
+                if (r < p.m) {
+                    const float xv = SeqT<DT>::ld(p.x, (size_t)r * p.ldx + k);
+#pragma unroll
+                    for (int c = 0; c < CPW; ++c) acc[r][c] = fmaf(wv[c], xv, acc[r][c]);
+                }
         }
     }
 #pragma unroll
-    for (int r = 0; r < MR; ++r) {
-        const float v = zl_wave_sum(acc[r]);
-        if (lane == 0 && r < p.m) SeqT<ODT>::st(p.y, (size_t)r * p.ldy + col, v);
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) {
+            const float v = zl_wave_sum(acc[r][c]);
+            if (lane == 0 && r < p.m && col0 + c < p.n) SeqT<ODT>::st(p.y, (size_t)r * p.ldy + col0 + c, v);
+        }
+}
+
+// 3 .. 16 activation rows in bf16 on the matrix cores without LDS staging: a workgroup owns 16 output columns, its four waves take every
+// fourth 32-k step; per step a lane loads 16 bytes of ITS weight row (A operand: lane = column, 8 consecutive k) and 16 bytes of ITS
+// activation row (B operand: lane = row; rows past m are zero), eight steps in flight, one v_mfma_f32_16x16x32_bf16 each.  The weights are
+// read exactly once, the activations cost half the weight bytes at 8 rows (L2), and no VALU multiply is spent.  The four partial tiles
+// meet in LDS.
+template <int ODT>
+__global__ __launch_bounds__(256) void k_seq_gemv_mfma(const GemmP p) {
+    __shared__ float red[4][16][17];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nrow = lane & 15, kq = lane >> 4;
+    const int col0 = blockIdx.x * 16;
+    const uint16_t* wp = reinterpret_cast<const uint16_t*>(p.w) + (size_t)min(col0 + nrow, p.n - 1) * p.k + 8 * kq;
+    const bool xok = nrow < p.m;
+    const uint16_t* xp = reinterpret_cast<const uint16_t*>(p.x) + (size_t)(xok ? nrow : 0) * p.ldx + 8 * kq;
+    f4 acc = (f4){0.f, 0.f, 0.f, 0.f};
+    const int steps = (p.k + 31) / 32;
+    constexpr int U = 8;
+    for (int s0 = wave; s0 < steps; s0 += 4 * U) {
+        uint4 wf[U], xf[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k0 = 32 * (s0 + 4 * u);
+            const bool ok = k0 + 8 * kq < p.k;                          // (k is a multiple of 8: a lane's 8 values are all in or all out)
+            wf[u] = ok ? zl_load_nt(reinterpret_cast<const uint4*>(wp + k0)) : make_uint4(0, 0, 0, 0);
+            xf[u] = (ok && xok) ? *reinterpret_cast<const uint4*>(xp + k0) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, wf[u]), __builtin_bit_cast(b8, xf[u]), acc, 0, 0, 0);
     }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][4 * kq + r][nrow] = acc[r];   // acc[r] = sum for column col0 + 4 kq + r, row nrow
+    __syncthreads();
+    const int c = threadIdx.x >> 4, m = threadIdx.x & 15;
+    if (m < p.m && col0 + c < p.n)
+        SeqT<ODT>::st(p.y, (size_t)m * p.ldy + col0 + c, red[0][c][m] + red[1][c][m] + red[2][c][m] + red[3][c][m]);
 }
 
 // 128 x 128 tiles (four times the MFMAs per LDS fragment) when they still fill the chip, 64 x 64 otherwise
@@ -225,11 +280,16 @@ void launch_tiled(const GemmP& p, hipStream_t hs) {
 
 template <int DT, int ODT>
 int launch(const GemmP& p, hipStream_t hs) {
+    if constexpr (DT == ZL_BF16) {
+        if (p.m >= 3 && p.m <= 16 && p.vec && (p.k & 7) == 0) {
+            hipLaunchKernelGGL((k_seq_gemv_mfma<ODT>), dim3((unsigned)((p.n + 15) / 16)), dim3(256), 0, hs, p);
+            return zl_launch_status();
+        }
+    }
     if (p.m <= 8) {
-        const dim3 grid((unsigned)((p.n + 3) / 4));
-        if (p.m <= 2) hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 2>), grid, dim3(256), 0, hs, p);
-        else if (p.m <= 4) hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 4>), grid, dim3(256), 0, hs, p);
-        else hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 8>), grid, dim3(256), 0, hs, p);
+        if (p.m <= 2) hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 2, 1>), dim3((unsigned)((p.n + 3) / 4)), dim3(256), 0, hs, p);
+        else if (p.m <= 4) hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 4, 2>), dim3((unsigned)((p.n + 7) / 8)), dim3(256), 0, hs, p);
+        else hipLaunchKernelGGL((k_seq_gemv<DT, ODT, 8, 4>), dim3((unsigned)((p.n + 15) / 16)), dim3(256), 0, hs, p);
     } else {
         launch_tiled<DT, ODT>(p, hs);
     }
