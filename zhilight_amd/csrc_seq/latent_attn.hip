@@ -300,9 +300,13 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
     for (int dt = 0; dt < DV; ++dt) o[dt] = (fa_f4){0.f, 0.f, 0.f, 0.f};
     float m = p.sink ? p.sink[h] : -INFINITY, l = p.sink ? 1.0f : 0.0f;
 
-    for (int j0 = 0; j0 <= block_last; j0 += 64) {
-        __syncthreads();
-        for (int idx = tid; idx < 64 * DK * 4; idx += 256) {                       // K tile: 64 keys x (DK * 32) columns, zero past dim
+    // K and V^T tiles: the NEXT tile's 16-byte loads are issued into registers before the current tile's MFMAs and written to LDS after them
+    constexpr int KU = DK, VU = (DV + 1) / 2;                                      // 16-byte units per thread: 64 DK 4 / 256 and DV 16 8 / 256
+    uint4 kreg[KU], vreg[VU];
+    auto fetch_tiles = [&](int j0) {
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+            const int idx = tid + 256 * u;
             const int key = idx / (DK * 4), d = (idx % (DK * 4)) * 8;
             const uint16_t* src = p.k + (size_t)(cs + j0 + key) * p.ldk + (size_t)h * p.dim + d;
             uint4 v = make_uint4(0, 0, 0, 0);
@@ -313,15 +317,35 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
                 for (int i = 0; i < 8; ++i) e[i] = d + i < p.dim ? src[i] : (uint16_t)0;
                 v = make_uint4(e[0] | (uint32_t)e[1] << 16, e[2] | (uint32_t)e[3] << 16, e[4] | (uint32_t)e[5] << 16, e[6] | (uint32_t)e[7] << 16);
             }
-            *reinterpret_cast<uint4*>(Ks + key * KR + d) = v;
+            kreg[u] = v;
         }
-        for (int idx = tid; idx < DV * 16 * 8; idx += 256) {                       // V^T tile: (DV * 16) rows x 64 keys, zero past vdim
+#pragma unroll
+        for (int u = 0; u < VU; ++u) {
+            const int idx = tid + 256 * u;
             const int d = idx >> 3, c8 = (idx & 7) * 8;
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (d < p.vdim) v = *reinterpret_cast<const uint4*>(p.vt + ((size_t)h * p.vdim + d) * p.ldv + cs + j0 + c8);
-            *reinterpret_cast<uint4*>(Vs + d * VR + c8) = v;
+            if (idx < DV * 16 * 8 && d < p.vdim) v = *reinterpret_cast<const uint4*>(p.vt + ((size_t)h * p.vdim + d) * p.ldv + cs + j0 + c8);
+            vreg[u] = v;
         }
+    };
+    auto publish_tiles = [&]() {
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+            const int idx = tid + 256 * u;
+            *reinterpret_cast<uint4*>(Ks + (idx / (DK * 4)) * KR + (idx % (DK * 4)) * 8) = kreg[u];
+        }
+#pragma unroll
+        for (int u = 0; u < VU; ++u) {
+            const int idx = tid + 256 * u;
+            if (idx < DV * 16 * 8) *reinterpret_cast<uint4*>(Vs + (idx >> 3) * VR + (idx & 7) * 8) = vreg[u];
+        }
+    };
+    fetch_tiles(0);
+    for (int j0 = 0; j0 <= block_last; j0 += 64) {
+        __syncthreads();                                                           // the previous tile is consumed
+        publish_tiles();
         __syncthreads();
+        if (j0 + 64 <= block_last) fetch_tiles(j0 + 64);                           // in flight during this tile's MFMAs
         if (j0 > wave_last) continue;                                              // wave-uniform; the barriers above stay in step
         fa_f4 sc[4];
         float mx = -INFINITY;
