@@ -83,10 +83,11 @@ int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* w
 int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* w_uk,
                          const void* w_uv, const float* sink, const void* cache, const zls_batch_t* b, float scale, int64_t heads,
                          int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, void* workspace, int64_t n_splits,
-                         zl_stream_t s);
+                         int no_mfma, zl_stream_t s);
 int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t heads, int64_t rank, int64_t n_splits);
 /* The keys of every token are split over n_splits workgroups (the caller picks it so that the launch fills the chip; any value >= 1 is
- * valid) whose partial results go through `workspace`; rank <= 1024.  single_only != 0: only sequences that bring ONE token are served (their rows of out written); portions are left to
+ * valid) whose partial results go through `workspace`; rank <= 1024.  In bf16 with rank % 8 == 0 and rank <= 512 the split pass runs
+ * on the matrix cores unless no_mfma != 0 (then, and otherwise, an fp32 VALU kernel).  single_only != 0: only sequences that bring ONE token are served (their rows of out written); portions are left to
  * zls_latent_attention_prompt.
  *
  * The same attention for PORTIONS (more than one token) on the matrix cores, bf16 only, over keys and values that the caller has

@@ -109,8 +109,9 @@ def mixer_sd(cfg, i, seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("portions", [[150], [2, 61, 1, 1, 64, 21], [63, 2, 85]])
-def test_latent_attention_alone(dev, dtype, portions):
+@pytest.mark.parametrize("portions", [[150], [2, 61, 1, 1, 64, 21], [63, 2, 85], [1] * 40 + [3] + [1] * 70])
+@pytest.mark.parametrize("kernels", ["matrix cores", "plain"])
+def test_latent_attention_alone(dev, dtype, portions, kernels):
     from zhilight_amd.cache import CacheManager
     from zhilight_amd.mixers import LatentAttention
     cfg = O.small_config(("latent_attention",))
@@ -122,6 +123,7 @@ def test_latent_attention_alone(dev, dtype, portions):
     cache = CacheManager(256, 2, dev)
     mix = LatentAttention("a", W, m["heads"], m["dim"], m["vdim"], m["kv_rank"], m["scale"], 1e-5).load(lambda n: sub[n], "", dtype, dev)
     mix.bind(cache, dtype)
+    mix.prompt_kernel = mix.decode_mfma = kernels == "matrix cores"     # (bf16 only; fp32 serving has the one plain kernel)
     cache.admit("s")
     got, at = [], 0
     for n in portions:

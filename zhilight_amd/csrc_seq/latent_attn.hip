@@ -426,6 +426,138 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
         }
 }
 
+// ---- single tokens in bf16 on the matrix cores --------------------------------------------------------------------------------------
+// One wave = one token x 16 heads x one split of the keys.  Per 32 keys: the latent rows go from the pages straight into A operands
+// (lane = key, 8 consecutive latent columns per 16-byte load), S^T (16 keys x 16 heads) = C . Q'^T with the folded queries as B operands
+// held in registers; softmax per lane (= per head) as in the prompt kernel; the rows are then parked in LDS and read back column-wise for
+// O^T (latent x 16 heads) += C^T . P^T (the contraction runs over the 32 keys in the order the scores lie in the lanes; two bf16 halves
+// per weight).  Leaves (max, denominator, sums) per split in the workspace of k_latent_split's format: k_latent_combine finishes both.
+template <int RT>                                                                  // rank <= 32 RT
+__global__ __launch_bounds__(64) void k_latent_decode_mfma(const AttnP p, const zls_batch_t b, const float* __restrict__ qa,
+                                                           float* __restrict__ ws, int n_splits) {
+    constexpr int CR = RT * 32 + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t ct[32 * CR];
+    const int t = blockIdx.x, split = blockIdx.z, lane = threadIdx.x, nrow = lane & 15, kq = lane >> 4;
+    const int head = blockIdx.y * 16 + nrow;
+    const bool hvalid = head < p.heads;
+    const int sq = b.tok_seq[t];
+    if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;
+    const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
+    const int nkeys = pos + 1;
+    const int chunk = ((nkeys + n_splits - 1) / n_splits + 31) & ~31;
+    const int k0 = split * chunk, k1 = min(nkeys, k0 + chunk);
+    const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
+    const uint16_t* cache = reinterpret_cast<const uint16_t*>(p.cache);
+
+    uint4 qf[RT];
+    {
+        const float* qr = qa + ((size_t)t * p.heads + (hvalid ? head : 0)) * p.rank;
+#pragma unroll
+        for (int kk = 0; kk < RT; ++kk) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = 32 * kk + 8 * kq + 2 * i;
+                const float a = (hvalid && r < p.rank) ? qr[r] : 0.f, c = (hvalid && r + 1 < p.rank) ? qr[r + 1] : 0.f;
+                w[i] = ZT<ZL_BF16>::from_f32(a) | (uint32_t)ZT<ZL_BF16>::from_f32(c) << 16;
+            }
+            qf[kk] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+    fa_f4 o[2 * RT];
+#pragma unroll
+    for (int rt = 0; rt < 2 * RT; ++rt) o[rt] = (fa_f4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int j0 = k0; j0 < k1; j0 += 32) {
+        uint4 cr[2][RT];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int j = j0 + 16 * c + nrow;
+            const bool valid = j < k1;
+            const size_t base = valid ? ((size_t)pages[j / b.page_size] * b.page_size + j % b.page_size) * p.rank : 0;
+#pragma unroll
+            for (int kk = 0; kk < RT; ++kk) {
+                const int r = 32 * kk + 8 * kq;
+                cr[c][kk] = (valid && r < p.rank) ? *reinterpret_cast<const uint4*>(cache + base + r) : make_uint4(0, 0, 0, 0);
+            }
+        }
+        fa_f4 sc[2];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            sc[c] = (fa_f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < RT; ++kk)
+                sc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(fa_b8, cr[c][kk]), __builtin_bit_cast(fa_b8, qf[kk]), sc[c], 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float v = (j0 + 16 * c + 4 * kq + r < k1) ? sc[c][r] : -INFINITY;        // (the folded query carries the scale)
+                sc[c][r] = v;
+                mx = fmaxf(mx, v);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mnew = fmaxf(m, mx);                                           // finite: key j0 is valid
+        const float corr = expf(m - mnew);                                         // m = -inf at the first block: 0
+        float ps = 0.f;
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+#pragma unroll
+            for (int r = 0; r < 4; r += 2) {
+                uint16_t hb[2], lb[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float pv = sc[c][r + e] == -INFINITY ? 0.f : expf(sc[c][r + e] - mnew);
+                    ps += pv;
+                    hb[e] = ZT<ZL_BF16>::from_f32(pv);
+                    lb[e] = ZT<ZL_BF16>::from_f32(pv - ZT<ZL_BF16>::to_f32(hb[e]));
+                }
+                hi[2 * c + (r >> 1)] = hb[0] | (uint32_t)hb[1] << 16;
+                lo[2 * c + (r >> 1)] = lb[0] | (uint32_t)lb[1] << 16;
+            }
+        }
+        ps += __shfl_xor(ps, 16, 64);
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * corr + ps;
+        m = mnew;
+        const fa_b8 ph = __builtin_bit_cast(fa_b8, make_uint4(hi[0], hi[1], hi[2], hi[3]));
+        const fa_b8 pl = __builtin_bit_cast(fa_b8, make_uint4(lo[0], lo[1], lo[2], lo[3]));
+        __syncthreads();                                                           // the previous block's column reads are done
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int kk = 0; kk < RT; ++kk) *reinterpret_cast<uint4*>(ct + (16 * c + nrow) * CR + 32 * kk + 8 * kq) = cr[c][kk];
+        __syncthreads();
+#pragma unroll
+        for (int rt = 0; rt < 2 * RT; ++rt) {
+            // slot s of lane group kq <-> key 16 (s / 4) + 4 kq + s % 4 of the block; this lane's column of the latent: 16 rt + nrow
+            uint32_t w[4];
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) {
+                const int ka = 16 * (s2 >> 1) + 4 * kq + 2 * (s2 & 1);
+                w[s2] = ct[ka * CR + 16 * rt + nrow] | (uint32_t)ct[(ka + 1) * CR + 16 * rt + nrow] << 16;
+            }
+            const fa_b8 a = __builtin_bit_cast(fa_b8, make_uint4(w[0], w[1], w[2], w[3]));
+            o[rt] *= corr;
+            o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ph, o[rt], 0, 0, 0);
+            o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pl, o[rt], 0, 0, 0);
+        }
+    }
+    if (!hvalid) return;
+    float* out = ws + (((size_t)t * p.heads + head) * n_splits + split) * (p.rank + 2);
+    if (kq == 0) { out[0] = m; out[1] = l; }
+#pragma unroll
+    for (int rt = 0; rt < 2 * RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 16 * rt + 4 * kq + i;
+            if (r < p.rank) out[2 + r] = o[rt][i];
+        }
+}
+
 }  // namespace
 
 extern "C" int zls_latent_store(const float* proj, int64_t ld, int64_t col0, const float* weight, float eps, int64_t rank, const zls_batch_t* b,
@@ -446,7 +578,7 @@ extern "C" int64_t zls_latent_attention_workspace_bytes(int64_t n_tok, int64_t h
 extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0, const float* gate, int64_t ldg, int64_t g_col0, const void* w_uk,
                                     const void* w_uv, const float* sink, const void* cache, const zls_batch_t* b, float scale, int64_t heads,
                                     int64_t dim, int64_t vdim, int64_t rank, void* out, int dtype, int single_only, void* workspace,
-                                    int64_t n_splits, zl_stream_t s) {
+                                    int64_t n_splits, int no_mfma, zl_stream_t s) {
     ZL_CHECK_ARG(q && w_uk && w_uv && cache && out && workspace && seq_batch_ok(b) && b->page_table && b->page_size > 0 && b->max_pages > 0, ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && dim > 0 && vdim > 0 && rank > 0 && heads <= 65535 && n_splits > 0 && n_splits <= 65535, ZL_EINVAL);
     ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && (!gate || (g_col0 >= 0 && g_col0 + heads <= ldg)), ZL_ESHAPE);
@@ -462,10 +594,19 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
     float* ws = (float*)workspace;
     float* qa = ws + (size_t)b->n_tok * heads * n_splits * (rank + 2);
     const int ns = (int)n_splits;
+    // bf16 with aligned rows of at most 512 latent columns: the split pass on the matrix cores (absorb and combine are shared)
+    const bool mfma = dtype == ZL_BF16 && p.vec && rank <= 512 && !no_mfma;
+    const dim3 mgrid(b->n_tok, (unsigned)((heads + 15) / 16), (unsigned)n_splits);
+#define MSPLIT(RT) hipLaunchKernelGGL((k_latent_decode_mfma<RT>), mgrid, dim3(64), 0, hs, p, *b, qa, ws, ns)
 #define SPLIT(DT, RPL) hipLaunchKernelGGL((k_latent_split<DT, RPL>), grid, dim3(256), lds, hs, p, *b, qa, ws, ns)
 #define CALL(DT)                                  \
     hipLaunchKernelGGL((k_latent_absorb<DT>), dim3(b->n_tok, (unsigned)heads, (unsigned)((rank + 63) / 64)), dim3(256), 0, hs, p, *b, qa); \
-    if (rank <= 64) SPLIT(DT, 1);                 \
+    if (mfma) {                                   \
+        if (rank <= 64) MSPLIT(2);                \
+        else if (rank <= 128) MSPLIT(4);          \
+        else if (rank <= 256) MSPLIT(8);          \
+        else MSPLIT(16);                          \
+    } else if (rank <= 64) SPLIT(DT, 1);          \
     else if (rank <= 128) SPLIT(DT, 2);           \
     else if (rank <= 256) SPLIT(DT, 4);           \
     else if (rank <= 512) SPLIT(DT, 8);           \
@@ -474,6 +615,7 @@ extern "C" int zls_latent_attention(const float* q, int64_t ldq, int64_t q_col0,
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
 #undef SPLIT
+#undef MSPLIT
     return zl_launch_status();
 }
 

@@ -43,6 +43,7 @@ class LatentAttention:
         self.scale, self.eps, self.has_sink, self.has_gate = float(scale), float(eps), sink, gate
         self.cache = None
         self.prompt_kernel = True         # bf16 portions on the matrix-core kernel (False: everything on the latent-space kernel)
+        self.decode_mfma = True           # bf16 single tokens: the split pass on the matrix cores (False: the fp32 VALU kernel)
 
     def load(self, get, prefix, dtype, device):
         H, d, v, r, W = self.heads, self.dim, self.vdim, self.rank, self.width
@@ -91,7 +92,7 @@ class LatentAttention:
             seqops.latent_attention_prompt(proj, 0, gate, H * d + r, k, vt, self.sink, batch, self.scale, H, d, self.vdim, a)
         if not prompt or batch.n_single:
             seqops.latent_attention(proj, 0, gate, H * d + r, self.w_uk, self.w_uv, self.sink, self.cache, batch, self.scale, H, d, self.vdim,
-                                    out=a, single_only=prompt)
+                                    out=a, single_only=prompt, mfma=self.decode_mfma)
         return seqops.gemm_nt(a, self.w_o)
 
 

@@ -239,7 +239,7 @@ def latent_attention_prompt(q, q_col0, gate, g_col0, k, vt, sink, batch, scale, 
     return out
 
 
-def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim, out=None, single_only=False):
+def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim, out=None, single_only=False, mfma=True):
     _cuda(q, gate, w_uk, w_uv, sink, cache)
     _f32(q, gate, sink)
     rank = cache.shape[2]
@@ -256,7 +256,7 @@ def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, sc
                      dtype=torch.float32, device=cache.device)
     check(lib().zls_latent_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _p(w_uk),
                                      _p(w_uv), _p(sink), _p(cache), batch.ref, _f(scale), _i(heads), _i(dim), _i(vdim), _i(rank), _p(out),
-                                     C.c_int(dt_code(cache.dtype)), C.c_int(int(single_only)), _p(ws), _i(n_splits), _stream()),
+                                     C.c_int(dt_code(cache.dtype)), C.c_int(int(single_only)), _p(ws), _i(n_splits), C.c_int(0 if mfma else 1), _stream()),
           "latent_attention")
     return out
 
