@@ -373,3 +373,43 @@ def test_seeded_sampling_is_reproducible_and_respects_top_k(dev, case):
     for i, t in enumerate(o):
         row = full[len(p) - 1 + i]
         assert t in torch.topk(row, 6).indices.tolist()
+
+
+MEDIUM = {
+    "a": dict(width=256, vocab=300, att=dict(dim=64, heads=6, kv_rank=160, scale=0.125, vdim=48),
+              ssm=dict(conv=4, groups=2, heads=8, norm_groups=2, state=128, vdim=64), ff=520, order="asa"),
+    "b": dict(width=384, vocab=520, att=dict(dim=128, heads=20, kv_rank=512, scale=0.09, vdim=128),
+              ssm=dict(conv=2, groups=3, heads=6, norm_groups=1, state=64, vdim=32), ff=1000, order="sas"),
+    "c": dict(width=200, vocab=210, att=dict(dim=40, heads=5, kv_rank=72, scale=0.2, vdim=72),
+              ssm=dict(conv=3, groups=1, heads=3, norm_groups=3, state=48, vdim=20), ff=264, order="aas"),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("name", sorted(MEDIUM))
+def test_medium_sizes_whole_chunked_and_decoded(dev, name, dtype):
+    """sizes that take the other instantiations of the kernels (head sizes 40 .. 128, ranks 72 .. 512, more than 16 heads, state-space heads of
+    20 .. 64 columns with 48 .. 128 states): a whole prompt, portions with single tokens between them, and a batch of two"""
+    from zhilight_amd.engine import Entry
+    z = MEDIUM[name]
+    layers = [{"type": "latent_attention" if ch == "a" else "mamba2", "mixer": dict(z["att"] if ch == "a" else z["ssm"]),
+               "mlp": None if i == 1 and name == "b" else {"ff": z["ff"], "kind": "dense"}} for i, ch in enumerate(z["order"])]
+    cfg = {"architecture": "Tupitar", "embedding": {"scale": 11.0}, "layers": layers, "max_positions": 400, "norm": {"eps": 1e-6},
+           "vocab": z["vocab"], "width": z["width"]}
+    sd = O.random_weights(cfg, seed=41)
+    toks, other = tokens_of(cfg, 150, 42), tokens_of(cfg, 70, 43)
+    ref, ref_other = O.forward(cfg, sd, toks), O.forward(cfg, sd, other)
+    eng = make(cfg, sd, dtype, dev, max_tokens=512)
+    assert rel(run_portions(eng, "w", toks, [150]), ref) < tol(dtype)
+    assert rel(run_portions(eng, "c", toks, [37, 1, 1, 30, 2, 65, 1, 13]), ref) < tol(dtype)
+    got = {"x": [], "y": []}
+    at = {"x": 0, "y": 0}
+    seqs = {"x": toks, "y": other}
+    for step in ([("x", 100), ("y", 3)], [("x", 1), ("y", 66)], [("x", 49), ("y", 1)]):
+        lg = eng.run_step([Entry(k, seqs[k][at[k]:at[k] + n], list(range(n))) for k, n in step])
+        row = 0
+        for k, n in step:
+            got[k].append(lg[row:row + n])
+            row += n
+            at[k] += n
+    assert rel(torch.cat(got["x"]), ref) < tol(dtype) and rel(torch.cat(got["y"]), ref_other) < tol(dtype)
