@@ -15,6 +15,11 @@ TP=1 replicas (one model + its own requests per GPU, no data-path collective), i
 `value` is the whole-job aggregate tokens/s.  Rank 0 prints ONE JSON line with, besides the contract
 fields, `roofline` (the W4A16 GEMV kernel: algorithmic bytes / HIP-event time, vs 8 TB/s HBM) and
 `cpu_baseline` (the CPU oracle timed on a bounded sample on this box's host cores).
+
+    python bench.py --mixers 1b,8b [--seq 2048]
+
+is a different measurement with its own JSON line: prefill / decode throughput of the ragged-step engine's latent-attention, state-space
+and hybrid stacks (zhilight_amd/tupitar.py) beside the dense bf16 Llama-shaped stack of equal width, 4 layers each, random weights.
 """
 import argparse
 import json
