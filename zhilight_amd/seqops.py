@@ -239,7 +239,8 @@ def latent_attention_prompt(q, q_col0, gate, g_col0, k, vt, sink, batch, scale, 
     return out
 
 
-def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim, out=None, single_only=False, mfma=True):
+def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, scale, heads, dim, vdim, out=None, single_only=False, mfma=True,
+                     n_splits=None):
     _cuda(q, gate, w_uk, w_uv, sink, cache)
     _f32(q, gate, sink)
     rank = cache.shape[2]
@@ -251,7 +252,8 @@ def latent_attention(q, q_col0, gate, g_col0, w_uk, w_uv, sink, cache, batch, sc
         out = torch.empty((batch.n_tok, heads * vdim), dtype=cache.dtype, device=cache.device)
     # enough workgroups to fill the chip (256 CUs, a few per CU), at least 64 keys per split
     groups = batch.n_tok * ((heads + 3) // 4)
-    n_splits = max(1, min((batch.max_ctx + 63) // 64, (1024 + groups - 1) // groups))
+    if n_splits is None:
+        n_splits = max(1, min((batch.max_ctx + 63) // 64, (1024 + groups - 1) // groups))
     ws = torch.empty(int(lib().zls_latent_attention_workspace_bytes(_i(batch.n_tok), _i(heads), _i(rank), _i(n_splits))) // 4,
                      dtype=torch.float32, device=cache.device)
     check(lib().zls_latent_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _p(w_uk),
