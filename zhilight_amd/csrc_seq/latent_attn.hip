@@ -2,13 +2,14 @@
 //
 // Beside csrc/mla_attn.hip (DeepSeek's geometry: 512 + 64 rotated columns, 16-bit, decode rows only, no sink): this one has no rotated
 // part, any rank / head sizes, a learned per-head sink in the softmax denominator, a per-head sigmoid output gate, causal portions of
-// prompts at any offset, and a 32-bit mode.  Only the latent is cached; keys and values are never materialised:
+// prompts at any offset, and a 32-bit mode.  Only the latent is cached; for single tokens keys and values are never materialised:
 //     score_j = (W_uk,h^T q_h) . c_j * scale          o_h = W_uv,h . (sum_j w_j c_j)
-// k_latent_store   RMS norm (plain weight) of the down-projection -> the token's cache row
-// k_latent_split   single tokens (and, in 32-bit serving, every token): the query is folded through W_uk, the keys are split over
-//                  workgroups, fp32 VALU; k_latent_combine merges the splits with the sink (it counts once, unscaled, with no value),
-//                  applies W_uv and the gate.
-// k_latent_fa      portions of prompts in bf16 on the matrix cores, over up-projected keys and values.
+// k_latent_store        RMS norm (plain weight) of the down-projection -> the token's cache row
+// k_latent_absorb       the query folded through W_uk (and the scale), once per token and head
+// k_latent_split        single tokens (and, in 32-bit serving, every token): the keys split over workgroups, fp32 VALU
+// k_latent_decode_mfma  the same split pass for bf16 on the matrix cores
+// k_latent_combine      merges the splits with the sink (it counts once, unscaled, with no value), applies W_uv and the gate
+// k_latent_fa           portions of prompts in bf16 on the matrix cores, over keys and values up-projected for the step
 #include "seq_common.h"
 
 namespace {
