@@ -269,7 +269,8 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
     constexpr int KR = DK * 32 + 8, VR = 64 + 8;
     __shared__ __attribute__((aligned(16))) uint16_t Ks[64 * KR];
     __shared__ __attribute__((aligned(16))) uint16_t Vs[DV * 16 * VR];
-    const int sq = blockIdx.x / p.tiles_per_seq, tile = blockIdx.x % p.tiles_per_seq, h = blockIdx.y;
+    // (the last query tiles see the most keys: they are dispatched first, so the launch does not end on its longest workgroups)
+    const int sq = blockIdx.x % b.n_seq, tile = p.tiles_per_seq - 1 - blockIdx.x / b.n_seq, h = blockIdx.y;
     const int first = b.seq_start[sq], count = b.seq_start[sq + 1] - first;
     const int cs = p.ctx_start[sq];
     if (cs < 0 || tile * 64 >= count) return;
