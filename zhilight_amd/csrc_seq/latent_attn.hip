@@ -252,10 +252,19 @@ __global__ __launch_bounds__(256) void k_latent_combine(const AttnP p, const zls
 //   blocks side by side are a B operand of the same instruction with the 32 keys in a permuted order, and V^T is read in that order too,
 //   so the weights never travel through LDS:
 //   O^T (vdim x 16 queries) += V^T_tile . P^T, with P = hi + lo (two bf16 halves: the weights keep 16 bits of mantissa).
-// Scores, running maximum / denominator (starting at the sink: m = sink, l = 1) and the output sums are fp32, per lane = per query.
+// Scores, running maximum / denominator (starting at the sink: m = sink, l = 1) and the output sums are fp32, per lane = per query; the
+// exponentials are the hardware's exp2 of the fp32 argument times log2 e (the softmax VALU work, not the MFMAs, bounds this kernel).
 typedef __bf16 fa_b8 __attribute__((ext_vector_type(8)));
 typedef short fa_s4 __attribute__((ext_vector_type(4)));
 typedef float fa_f4 __attribute__((ext_vector_type(4)));
+
+// a non-negative fp32 weight as two bf16 halves, hi + lo = the weight to 2^-16 relative: hi is its upper 16 bits (truncation), lo the upper
+// 16 bits of the exact remainder -- three instructions where two round-to-nearest conversions cost a dozen
+__device__ __forceinline__ void fa_split(float pv, uint16_t& hb, uint16_t& lb) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, pv);
+    hb = (uint16_t)(u >> 16);
+    lb = (uint16_t)(__builtin_bit_cast(uint32_t, pv - __builtin_bit_cast(float, u & 0xffff0000u)) >> 16);
+}
 
 struct FaP {
     const float* q; const float* gate; const uint16_t* k; const uint16_t* vt; const float* sink; const int32_t* ctx_start; uint16_t* out;
@@ -373,7 +382,7 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mnew = fmaxf(m, mx);
         const bool dead = mnew == -INFINITY;                                       // nothing seen yet and no sink: keep zeros
-        const float corr = dead ? 1.0f : expf(m - mnew);
+        const float corr = dead ? 1.0f : __expf(m - mnew);
         float ps = 0.f;
         // the 32-key contraction of v_mfma_f32_16x16x32_bf16 may run over the keys in ANY order as long as both operands use the same one:
         // slot s of lane group kq stands for key 16 (s / 4) + 4 kq + s % 4 of the pair of 16-key blocks, which is how the scores lie here
@@ -385,10 +394,9 @@ __global__ __launch_bounds__(256) void k_latent_fa(const FaP p, const zls_batch_
                 uint16_t hb[2], lb[2];
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    const float pv = (dead || sc[c][r + e] == -INFINITY) ? 0.f : expf(sc[c][r + e] - mnew);
+                    const float pv = (dead || sc[c][r + e] == -INFINITY) ? 0.f : __expf(sc[c][r + e] - mnew);
                     ps += pv;
-                    hb[e] = ZT<ZL_BF16>::from_f32(pv);
-                    lb[e] = ZT<ZL_BF16>::from_f32(pv - ZT<ZL_BF16>::to_f32(hb[e]));
+                    fa_split(pv, hb[e], lb[e]);
                 }
                 hi[c >> 1][2 * (c & 1) + (r >> 1)] = hb[0] | (uint32_t)hb[1] << 16;
                 lo[c >> 1][2 * (c & 1) + (r >> 1)] = lb[0] | (uint32_t)lb[1] << 16;
@@ -502,7 +510,7 @@ __global__ __launch_bounds__(64) void k_latent_decode_mfma(const AttnP p, const 
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mnew = fmaxf(m, mx);                                           // finite: key j0 is valid
-        const float corr = expf(m - mnew);                                         // m = -inf at the first block: 0
+        const float corr = __expf(m - mnew);                                       // m = -inf at the first block: 0
         float ps = 0.f;
         uint32_t hi[4], lo[4];
 #pragma unroll
@@ -512,10 +520,9 @@ __global__ __launch_bounds__(64) void k_latent_decode_mfma(const AttnP p, const 
                 uint16_t hb[2], lb[2];
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    const float pv = sc[c][r + e] == -INFINITY ? 0.f : expf(sc[c][r + e] - mnew);
+                    const float pv = sc[c][r + e] == -INFINITY ? 0.f : __expf(sc[c][r + e] - mnew);
                     ps += pv;
-                    hb[e] = ZT<ZL_BF16>::from_f32(pv);
-                    lb[e] = ZT<ZL_BF16>::from_f32(pv - ZT<ZL_BF16>::to_f32(hb[e]));
+                    fa_split(pv, hb[e], lb[e]);
                 }
                 hi[2 * c + (r >> 1)] = hb[0] | (uint32_t)hb[1] << 16;
                 lo[2 * c + (r >> 1)] = lb[0] | (uint32_t)lb[1] << 16;
