@@ -126,6 +126,100 @@ int64_t zls_ssm_scan_workspace_bytes(int64_t n_seq, int64_t max_count, int64_t s
 int zls_gated_group_norm(const float* y, const float* proj, int64_t ld, int64_t z_col0, const float* weight, float eps, int64_t rows,
                          int64_t inner, int64_t norm_groups, void* out, int dtype, zl_stream_t s);
 
+/* ---- layer norm --------------------------------------------------------------------------------------------------------------- */
+/* out[i] = (x[r] - mean) / sqrt(var + eps) * w + b with r = rows[i] (rows NULL: r = i), var = mean of the squared deviations; x fp32
+ * (.., width), w, b fp32 (width; b nullable), out (n_rows, width) in `dtype`.  Both moments are fp32, the mean taken first. */
+int zls_layer_norm(const float* x, const int32_t* rows, const float* w, const float* b, float eps, int64_t n_rows, int64_t width, void* out,
+                   int dtype, zl_stream_t s);
+/* x[t] += layer_norm(y[t]; w, b) in place (x, y fp32 (rows, width)); with w2 (nullable, then b2 nullable too) also
+ * h2[t] = layer_norm(new x[t]; w2, b2) in `dtype`: the input of the next matrix product, from the same launch. */
+int zls_add_layer_norm(float* x, const float* y, const float* w, const float* b, float eps, int64_t rows, int64_t width, const float* w2,
+                       const float* b2, void* h2, int dtype, zl_stream_t s);
+
+/* ---- softmax attention over a paged key / value cache: rotary positions, unit-RMS queries and keys, turned values, a sliding window,
+ *      weights mixed across heads ------------------------------------------------------------------------------------------------- */
+/* Per token at position p, in place on the fp32 projection row proj[t] (ld floats):
+ *   queries (heads x dim from q_col0) and keys (kv_heads x dim from k_col0): coordinate i < rot_dims / 2 of a head is paired with
+ *   i + rot_dims / 2 and the pair (u, v) becomes (u cos a - v sin a, v cos a + u sin a), a = p * qk_freq[i]; the other coordinates stay;
+ *   with qk_norm != 0 every head is then divided by sqrt(mean(head^2) + eps);
+ *   values (kv_heads x vdim from v_col0): with v_freq (nullable) turned the same way over ALL vdim coordinates, a = p * v_freq[i].
+ * Queries are written back to proj; keys and values go to the token's row of k_cache (pages, page_size, kv_heads * dim) and v_cache
+ * (pages, page_size, kv_heads * vdim) in `dtype`.  k_cache NULL (then v_cache too): only the queries are served -- a layer that reads
+ * another layer's cache.  qk_freq fp32 (rot_dims / 2; rot_dims even, <= dim; 0: no rotation), v_freq fp32 (vdim / 2; vdim even).
+ * dim, vdim <= 512. */
+int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int64_t heads, int64_t kv_heads, int64_t dim,
+                        int64_t vdim, const float* qk_freq, int64_t rot_dims, const float* v_freq, float eps, int qk_norm,
+                        const zls_batch_t* b, void* k_cache, void* v_cache, int dtype, zl_stream_t s);
+
+/* Softmax attention of every token over the cached keys j of its sequence with 0 <= p - j < window (window <= 0: all j <= p):
+ *   w_g(j) = softmax_j(scale * q_g . k_c(g)(j)),  c(g) = g / (heads / kv_heads)
+ *   all_kv == 0:  acc[t][g][:]    = sum_j w_g(j) v_c(g)(j)                      acc fp32 (n_tok, heads, vdim)
+ *   all_kv != 0:  acc[t][g][c][:] = sum_j w_g(j) v_c(j) for EVERY kv head c     acc fp32 (n_tok, heads, kv_heads, vdim)
+ * The second form is what mixing the heads' weights needs (zls_head_mix_gate): sum_j (sum_g T[h][g] w_g(j)) v_c(h)(j) =
+ * sum_g T[h][g] acc[g][c(h)].  q fp32 (n_tok, ldq) from q_col0 (as zls_rope_norm_store left it).  Scores, weights and sums are fp32; keys of a
+ * long context are walked in chunks with a running maximum.  (all_kv ? kv_heads : 1) * vdim <= 2048. */
+int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
+                         float scale, int64_t window, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc,
+                         int dtype, zl_stream_t s);
+
+/* out[t][h][:] = turn_back(sum_g talk[h][g] acc[t][g][c(h)][:]) * sigmoid(gate[t][h * vdim + :])
+ * talk fp32 (heads, heads), NULL: no mixing, acc is (n_tok, heads, vdim); v_freq (nullable): pair (m, m + vdim / 2) is turned by
+ * -p * v_freq[m]; gate fp32 (n_tok, ldg) from g_col0, NULL: no gate; out (n_tok, heads * vdim) in `dtype`. */
+int zls_head_mix_gate(const float* acc, const float* talk, const float* v_freq, const float* gate, int64_t ldg, int64_t g_col0,
+                      const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out, int dtype, zl_stream_t s);
+
+/* ---- linear attention with a scalar decay per head and token ---------------------------------------------------------------------- */
+/* S_t = a_t S_{t-1} + b_t k_t v_t^T,  y_t = S_t^T q_t   per head, S fp32 (dim x vdim) carried in state[slot].
+ *   q, k (heads x dim) and v (heads x vdim): columns q_col0 / k_col0 / v_col0 of the fp32 rows proj[t] (ld), passed through SiLU first when
+ *   act == 1;  a_t = decay_t[t][h] (fp32 (n_tok, heads)) or, with decay_t NULL, the constant decay_h[h];  b_t = gain_t[t][h] or 1.
+ *   norm_col != 0: the state has one more column that takes the value 1 for every token, i.e. holds n_t = a_t n_{t-1} + b_t k_t, and y
+ *   one more number per head, n_t . q_t.
+ * state fp32 (slots, heads, dim, vdim + norm_col); y fp32 (n_tok, heads * (vdim + norm_col)).  Long portions run in segments exactly as
+ * zls_ssm_scan's do (same kernel, workspace from zls_ssm_scan_workspace_bytes(n_seq, max_count, seg_len, heads, vdim + norm_col, dim)). */
+int zls_decay_scan(const float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int act, const float* decay_h,
+                   const float* decay_t, const float* gain_t, int norm_col, float* state, int64_t heads, int64_t dim, int64_t vdim,
+                   const zls_batch_t* b, float* y, void* workspace, int64_t seg_len, zl_stream_t s);
+
+/* Exponential gates with a running maximum (per sequence and head, tokens in order; m carried in m_state[slot][h], 0 for a new sequence):
+ *   i = cap tanh((zi + i_bias[h]) / cap),  f = log sigmoid(cap tanh((zf + f_bias[h]) / cap))      (cap <= 0: no cap)
+ *   m_t = max(f + m_{t-1}, i);  decay[t][h] = exp(f + m_{t-1} - m_t);  gain[t][h] = exp(i - m_t);  m_out[t][h] = m_t
+ * zi / zf = proj[t][i_col0 + h] / proj[t][f_col0 + h] (fp32, ld).  decay, gain, m_out fp32 (n_tok, heads). */
+int zls_exp_gates(const float* proj, int64_t ld, int64_t i_col0, int64_t f_col0, const float* i_bias, const float* f_bias, float cap,
+                  float* m_state, int64_t heads, const zls_batch_t* b, float* decay, float* gain, float* m_out, zl_stream_t s);
+
+/* The end of a linear-attention mixer: o = y[t][h][0 .. vdim) (row stride of a head: vdim + norm_col);
+ *   with m_vals (needs norm_col): o = q_scale * o / (max(|q_scale * y[t][h][vdim]|, exp(-m_vals[t][h])) + den_eps);
+ *   every one of `norm_groups` equal parts of the row heads * vdim is divided by sqrt(mean(part^2) + eps), times weight (nullable),
+ *   times sigmoid(gate[t][g_col0 + c]) (gate nullable).  out (n_tok, heads * vdim) in `dtype`. */
+int zls_linear_attn_finish(const float* y, int64_t norm_col, float q_scale, const float* m_vals, float den_eps, int64_t heads, int64_t vdim,
+                           int64_t norm_groups, const float* weight, float eps, const float* gate, int64_t ldg, int64_t g_col0,
+                           int64_t n_tok, void* out, int dtype, zl_stream_t s);
+
+/* ---- mixture of experts over a ragged step ------------------------------------------------------------------------------------------ */
+/* Router: s = softmax(logits[t]) over all n_out outputs; choice = s + correction (nullable); the outputs form `groups` equal groups of
+ * neighbours, a group's score is its largest choice score, only outputs of the `keep` best groups can be chosen (groups <= 1: all);
+ * the `top` largest choice scores are chosen (ties: the lower index).  ids int32 (n_tok, top), weights fp32 (n_tok, top) = s of the
+ * chosen (scaled by 1 / their sum when renorm != 0).  n_out <= 1024, n_out % groups == 0. */
+int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float* correction, int64_t groups, int64_t keep, int64_t top,
+                  int renorm, int32_t* ids, float* weights, zl_stream_t s);
+/* Sort the n_slots = n_tok * top (token, choice) pairs by expert: pairs whose id is >= n_experts (identity outputs) are left out.
+ *   sorted_tok[p] = token of the pair at sorted position p;  slot_pos[t * top + k] = p (or -1);
+ *   tiles[3 i ..] = (expert, first position, end position) of the i-th run of at most tile_m positions of one expert, expert = -1 for unused
+ *   entries up to max_tiles >= n_slots / tile_m + n_experts.  One workgroup. */
+int zls_moe_align(const int32_t* ids, int64_t n_slots, int64_t top, int64_t n_experts, int64_t tile_m, int32_t* sorted_tok, int32_t* slot_pos,
+                  int32_t* tiles, int64_t max_tiles, zl_stream_t s);
+/* y[p] = x[x_rows[p]] . w[expert of p]^T for every sorted position p: w (n_experts, n, k) in `dtype`, x_rows NULL: x[p]; `tiles` from
+ * zls_moe_align with tile_m = 64.  gated != 0: n = 2 ff rows per expert, stored as blocks of 16 gate rows followed by their 16 up rows
+ * (ff % 16 == 0), and y (.., ff) = silu(gate) * up in out_dtype.  Otherwise y (.., n). */
+int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, const int32_t* tiles, int64_t max_tiles, void* y,
+                        int64_t ldy, int64_t n, int64_t k, int gated, int dtype, int out_dtype, zl_stream_t s);
+/* out[p][c] = silu(gu[p][c]) * gu[p][ff + c]  for rows 0 .. rows - 1 (gu fp32 (rows, 2 ff)), out in `dtype`. */
+int zls_silu_mul(const float* gu, int64_t rows, int64_t ff, void* out, int dtype, zl_stream_t s);
+/* out[t] = sum_k weights[t][k] * (ids[t][k] >= n_experts ? h[t] : y[slot_pos[t * top + k]]), in the order of k; y fp32 (.., width),
+ * h (n_tok, width) in `dtype`, out fp32. */
+int zls_moe_combine(const float* y, const int32_t* slot_pos, const int32_t* ids, const float* weights, const void* h, int64_t n_tok,
+                    int64_t top, int64_t n_experts, int64_t width, float* out, int dtype, zl_stream_t s);
+
 #ifdef __cplusplus
 }
 #endif

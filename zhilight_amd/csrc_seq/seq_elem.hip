@@ -90,6 +90,43 @@ __global__ __launch_bounds__(kT) void k_polynorm(const float* __restrict__ z, fl
     }
 }
 
+// mean first, then the mean of the squared deviations (both fp32): the row is read three times, from L1 / L2 after the first
+__device__ __forceinline__ void ln_moments(const float* __restrict__ r, int width, float eps, float* red, float& mean, float& inv) {
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < width; i += kT) sum += r[i];
+    mean = zl_block_sum(sum, red) / (float)width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kT) { const float d = r[i] - mean; ss = fmaf(d, d, ss); }
+    inv = 1.0f / sqrtf(zl_block_sum(ss, red) / (float)width + eps);
+}
+
+template <int DT>
+__global__ __launch_bounds__(kT) void k_layer_norm(const float* __restrict__ x, const int32_t* __restrict__ rows, const float* __restrict__ w,
+                                                   const float* __restrict__ bias, float eps, int width, void* __restrict__ out) {
+    __shared__ float red[16];
+    const float* r = x + (size_t)(rows ? rows[blockIdx.x] : (int)blockIdx.x) * width;
+    const size_t orow = (size_t)blockIdx.x * width;
+    float mean, inv;
+    ln_moments(r, width, eps, red, mean, inv);
+    for (int i = threadIdx.x; i < width; i += kT) SeqT<DT>::st(out, orow + i, (r[i] - mean) * inv * w[i] + (bias ? bias[i] : 0.f));
+}
+
+// x += LN(y); optionally the NEXT sub-layer's input LN2(x) in the serving format from the same workgroup (the new row is in L1)
+template <int DT>
+__global__ __launch_bounds__(kT) void k_add_layer_norm(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w,
+                                                       const float* __restrict__ bias, float eps, int width, const float* __restrict__ w2,
+                                                       const float* __restrict__ bias2, void* __restrict__ h2) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * width;
+    float mean, inv;
+    ln_moments(y + row, width, eps, red, mean, inv);
+    for (int i = threadIdx.x; i < width; i += kT) x[row + i] += (y[row + i] - mean) * inv * w[i] + (bias ? bias[i] : 0.f);
+    if (!w2) return;
+    __syncthreads();                                             // (each thread re-reads rows that other threads wrote)
+    ln_moments(x + row, width, eps, red, mean, inv);
+    for (int i = threadIdx.x; i < width; i += kT) SeqT<DT>::st(h2, row + i, (x[row + i] - mean) * inv * w2[i] + (bias2 ? bias2[i] : 0.f));
+}
+
 }  // namespace
 
 extern "C" int zls_embed(const int32_t* tokens, const void* table, const void* pos_table, int64_t vocab, int64_t max_positions, float scale,
@@ -133,6 +170,24 @@ extern "C" int zls_scalar_norm_rows(const float* x, const int32_t* rows, float g
 extern "C" int zls_polynorm(const float* z, const float* coef, float eps, int64_t rows, int64_t ff, void* out, int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(z && coef && out && rows > 0 && ff > 0, ZL_EINVAL);
 #define CALL(DT) hipLaunchKernelGGL((k_polynorm<DT>), dim3((unsigned)rows), dim3(kT), 0, (hipStream_t)s, z, coef[0], coef[1], coef[2], coef[3], eps, (int)ff, out);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_layer_norm(const float* x, const int32_t* rows, const float* w, const float* b, float eps, int64_t n_rows, int64_t width,
+                              void* out, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(x && w && out && n_rows > 0 && width > 0, ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_layer_norm<DT>), dim3((unsigned)n_rows), dim3(kT), 0, (hipStream_t)s, x, rows, w, b, eps, (int)width, out);
+    ZLS_DISPATCH(dtype, CALL)
+#undef CALL
+    return zl_launch_status();
+}
+
+extern "C" int zls_add_layer_norm(float* x, const float* y, const float* w, const float* b, float eps, int64_t rows, int64_t width,
+                                  const float* w2, const float* b2, void* h2, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(x && y && w && rows > 0 && width > 0 && (!w2 || h2), ZL_EINVAL);
+#define CALL(DT) hipLaunchKernelGGL((k_add_layer_norm<DT>), dim3((unsigned)rows), dim3(kT), 0, (hipStream_t)s, x, y, w, b, eps, (int)width, w2, b2, h2);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();

@@ -24,6 +24,10 @@ struct GemmP {
     int m, n, k, vec;
     const int32_t* x_rows;                                     // row r of x is x[x_rows[r]] (NULL: r); the same for w
     const int32_t* w_rows;
+    // grouped form (a mixture of experts): row tile i of the launch is tiles[3 i ..] = (expert, first row, end row) with rows counted in
+    // the expert-sorted order, w = the expert's (n, k) block of a stacked (experts, n, k) array; expert < 0: the tile is unused
+    const int32_t* tiles;
+    int64_t w_stride;
 };
 
 // ---- tiles in LDS -----------------------------------------------------------------------------------------------------------------
@@ -66,7 +70,9 @@ template <> struct Tile<ZL_F32> {
 };
 
 // WT x WT MFMA tiles per wave: the workgroup's output tile is (32 WT) x (32 WT)
-template <int DT, int ODT, int WT>
+// GATED (WT = 2): the weight rows come in blocks of 16 gate rows followed by their 16 up rows, so that a wave's two column tiles are the gate
+// and the up projection of the same 16 outputs; the epilogue writes silu(gate) * up, half as many columns
+template <int DT, int ODT, int WT, bool GATED = false>
 __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
     typedef typename Tile<DT>::elem E;
     constexpr int RS = Tile<DT>::kRow;
@@ -76,7 +82,16 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nrow = lane & 15, kq = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
+    int m0 = blockIdx.y * kBM, mlim = p.m;
+    const int n0 = blockIdx.x * kBN;
+    const void* wbase = p.w;
+    if (p.tiles) {
+        const int e = p.tiles[3 * blockIdx.y];
+        if (e < 0) return;                                      // (the whole workgroup)
+        m0 = p.tiles[3 * blockIdx.y + 1];
+        mlim = p.tiles[3 * blockIdx.y + 2];
+        wbase = reinterpret_cast<const E*>(p.w) + (size_t)e * p.w_stride;
+    }
     const int lrow = tid >> 2, lkc = (tid & 3) * 8;
 
     f4 acc[WT][WT];
@@ -91,12 +106,12 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
 #pragma unroll
     for (int u = 0; u < PASS; ++u) {
         const int mr = m0 + lrow + 64 * u, nr = n0 + lrow + 64 * u;
-        xr[u] = (p.x_rows && mr < p.m) ? p.x_rows[mr] : mr;
+        xr[u] = (p.x_rows && mr < mlim) ? p.x_rows[mr] : mr;
         wr[u] = (p.w_rows && nr < p.n) ? p.w_rows[nr] : nr;
-        xlim[u] = mr < p.m ? xr[u] + 1 : 0;
+        xlim[u] = mr < mlim ? xr[u] + 1 : 0;
         wlim[u] = nr < p.n ? wr[u] + 1 : 0;
         tx[u].load(p.x, p.ldx, xr[u], xlim[u], 0, lkc, p.k, p.vec);
-        tw[u].load(p.w, p.ldw, wr[u], wlim[u], 0, lkc, p.k, p.vec);
+        tw[u].load(wbase, p.ldw, wr[u], wlim[u], 0, lkc, p.k, p.vec);
     }
     for (int k0 = 0; k0 < p.k; k0 += kBK) {
         __syncthreads();                                        // the previous slice's fragments are consumed
@@ -110,7 +125,7 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
 #pragma unroll
             for (int u = 0; u < PASS; ++u) {
                 tx[u].load(p.x, p.ldx, xr[u], xlim[u], k0 + kBK, lkc, p.k, p.vec);
-                tw[u].load(p.w, p.ldw, wr[u], wlim[u], k0 + kBK, lkc, p.k, p.vec);
+                tw[u].load(wbase, p.ldw, wr[u], wlim[u], k0 + kBK, lkc, p.k, p.vec);
             }
         }
         if constexpr (DT == ZL_BF16) {
@@ -139,6 +154,19 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
             }
         }
     }
+    if constexpr (GATED) {
+        static_assert(WT == 2, "the gated epilogue pairs a wave's two column tiles");
+        const int wcol = n0 + wn * 32 + nrow;                   // the gate's weight row; its output column is half the block offset
+        const int col = (n0 + wn * 32) / 2 + nrow;
+#pragma unroll
+        for (int i = 0; i < WT; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = m0 + wm * 32 + i * 16 + 4 * kq + r;
+                if (row < mlim && wcol < p.n) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, seq_silu(acc[i][0][r]) * acc[i][1][r]);
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < WT; ++i)
 #pragma unroll
@@ -147,7 +175,7 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = m0 + wm * 16 * WT + i * 16 + 4 * kq + r;
-                if (row < p.m && col < p.n) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, acc[i][j][r]);
+                if (row < mlim && col < p.n) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, acc[i][j][r]);
             }
         }
 }
@@ -309,7 +337,7 @@ extern "C" int zls_gemm_nt(const void* x, int64_t ldx, const void* w, void* y, i
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
     GemmP p;
     p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = k; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
-    p.x_rows = p.w_rows = nullptr;
+    p.x_rows = p.w_rows = nullptr; p.tiles = nullptr; p.w_stride = 0;
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
     p.vec = (k % unit == 0 && ldx % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
     hipStream_t hs = (hipStream_t)s;
@@ -328,7 +356,7 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
     GemmP p;
     p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.m = (int)m; p.n = (int)n; p.k = (int)k;
-    p.x_rows = x_rows; p.w_rows = w_rows;
+    p.x_rows = x_rows; p.w_rows = w_rows; p.tiles = nullptr; p.w_stride = 0;
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
     p.vec = (k % unit == 0 && ldx % unit == 0 && ldw % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
     hipStream_t hs = (hipStream_t)s;
@@ -338,5 +366,33 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
     } else {
         launch_tiled<ZL_F32, ZL_F32>(p, hs);
     }
+    return zl_launch_status();
+}
+
+// the grouped product of a mixture of experts: one launch over the (expert, row tile) list that zls_moe_align left on the device -- the host
+// never learns how many rows an expert got, the grid covers the upper bound and unused tiles return at once.  64-row tiles.
+extern "C" int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, const int32_t* tiles, int64_t max_tiles,
+                                   void* y, int64_t ldy, int64_t n, int64_t k, int gated, int dtype, int out_dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(x && w && tiles && y && max_tiles > 0 && n > 0 && k > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(ldx >= k && n < (1 << 30) && k < (1 << 30) && max_tiles <= 65535, ZL_ESHAPE);
+    ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
+    ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
+    ZL_CHECK_ARG(gated ? (n % 32 == 0 && ldy >= n / 2) : ldy >= n, ZL_ESHAPE);
+    GemmP p;
+    p.x = x; p.w = w; p.y = y; p.ldx = ldx; p.ldw = k; p.ldy = ldy; p.m = 0; p.n = (int)n; p.k = (int)k;
+    p.x_rows = x_rows; p.w_rows = nullptr; p.tiles = tiles; p.w_stride = n * k;
+    const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
+    p.vec = (k % unit == 0 && ldx % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
+    hipStream_t hs = (hipStream_t)s;
+    const dim3 grid((unsigned)((n + 63) / 64), (unsigned)max_tiles);
+#define GROUPED(DT, ODT)                                                                            \
+    if (gated) hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2, true>), grid, dim3(256), 0, hs, p);       \
+    else hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2, false>), grid, dim3(256), 0, hs, p);
+    if (dtype == ZL_BF16) {
+        if (out_dtype == ZL_F32) { GROUPED(ZL_BF16, ZL_F32) } else { GROUPED(ZL_BF16, ZL_BF16) }
+    } else {
+        GROUPED(ZL_F32, ZL_F32)
+    }
+#undef GROUPED
     return zl_launch_status();
 }

@@ -54,6 +54,11 @@ struct ScanP {
     // product of its decays (no y); 2 = a segment from its true start state (seg_init, or the slot's state for segment 0), writing y
     int mode, seg_len, n_seg;
     float* seg_state; float* seg_prod; float* seg_init;      // (n_seq, n_seg, heads, n_state, vdim) | (n_seq, n_seg, heads) | like seg_state
+    // kind 0: the Mamba-2 sources above.  kind 1: linear attention with a scalar decay -- the staged row [v | k | q] comes from columns of
+    // `proj` (x = v, B = k, C = q, each head its own), through SiLU when act is set; the input scale is gain_t[t][h] (or 1), the decay
+    // decay_t[t][h] (or the constant decay_h[h]); with `ones` the last of the vdim columns is not loaded but 1 for every token
+    int kind, act, ones, q_col0, k_col0, v_col0;
+    const float* decay_h; const float* decay_t; const float* gain_t;
 };
 
 constexpr int kScanSlots = 32;
@@ -76,8 +81,10 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
     const int sq = blockIdx.x / p.n_seg, seg = blockIdx.x % p.n_seg, h = blockIdx.y, tid = threadIdx.x, nthr = blockDim.x;
     const int pp = tid / p.ngl, g = tid % p.ngl;
     const bool active = pp < P;
-    const int grp = h / (p.heads / p.groups);
-    const int inner = p.heads * P, chan = inner + 2 * p.groups * N;
+    const bool lin = p.kind == 1;
+    const int grp = lin ? 0 : h / (p.heads / p.groups);
+    const int inner = p.heads * P, chan = lin ? (int)p.ld : inner + 2 * p.groups * N;
+    const float* srcbase = lin ? p.proj : p.xbc;
     const int whole = b.seq_start[sq + 1] - b.seq_start[sq];
     if (seg * p.seg_len >= whole) return;                               // (workgroup-uniform)
     const int first = b.seq_start[sq] + seg * p.seg_len, count = min(p.seg_len, whole - seg * p.seg_len);
@@ -93,7 +100,8 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
         S[j] = (p.mode != 1 && active && j < p.npt && n < N) ? init[(size_t)n * P + pp] : 0.f;
     }
     float prod = 1.0f;
-    const float rate = expf(p.a_log[h]), bias = p.dt_bias[h], dskip = p.d[h];
+    const float rate = lin ? 0.f : expf(p.a_log[h]), bias = lin ? 0.f : p.dt_bias[h], dskip = lin ? 0.f : p.d[h];
+    const float dec_h = (lin && !p.decay_t) ? p.decay_h[h] : 1.0f;
     // slot u of a thread = (token u / KP of the chunk, column e = tid + (u % KP) * threads of the staged row): where it comes from inside
     // xbc and where it goes in LDS is the same for every chunk, so both offsets are worked out once (a wave64 VALU instruction costs four
     // cycles and this loop runs at one wave per SIMD: index arithmetic per chunk would cost more than the recurrence itself)
@@ -101,32 +109,45 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
 #pragma unroll
     for (int u = 0; u < kScanSlots; ++u) {
         const int i = u / KP, e = tid + (u % KP) * nthr;
-        int col = h * P + e, at = e;
+        int col = lin ? p.v_col0 + h * (P - p.ones) + e : h * P + e, at = e;
         if (e >= P) {
             const int n = (e - P) % N, half = (e - P) / N;
-            col = inner + (half * p.groups + grp) * N + n;
+            col = lin ? (half ? p.q_col0 : p.k_col0) + h * N + n : inner + (half * p.groups + grp) * N + n;
             at = P4 + half * p.ngl * GS + (n / p.npt) * GS + n % p.npt;
         }
-        src_off[u] = e < W ? i * chan + col : -1;
+        src_off[u] = e < W ? ((lin && p.ones && e == P - 1) ? -2 : i * chan + col) : -1;      // -2: the column of ones
         dst_off[u] = i * WL + at;
     }
-    float pre[kScanSlots], pre_dt = 0.f;
+    float pre[kScanSlots], pre_dt = 0.f, pre_dec = 0.f;
     auto fetch = [&](int c0) {
         const int cn = min(CH, count - c0);
-        const float* base = p.xbc + (size_t)(first + c0) * chan;
+        const float* base = srcbase + (size_t)(first + c0) * chan;
 #pragma unroll
-        for (int u = 0; u < kScanSlots; ++u) pre[u] = (u < cn * KP && src_off[u] >= 0) ? base[src_off[u]] : 0.f;
-        if (tid < cn) pre_dt = p.proj[(size_t)(first + c0 + tid) * p.ld + p.dt_col0 + h];
+        for (int u = 0; u < kScanSlots; ++u) pre[u] = (u < cn * KP && src_off[u] >= 0) ? base[src_off[u]] : 1.0f;
+        if (tid < cn) {
+            if (lin) {
+                const size_t at = (size_t)(first + c0 + tid) * p.heads + h;
+                pre_dt = p.gain_t ? p.gain_t[at] : 1.0f;
+                pre_dec = p.decay_t ? p.decay_t[at] : dec_h;
+            } else {
+                pre_dt = p.proj[(size_t)(first + c0 + tid) * p.ld + p.dt_col0 + h];
+            }
+        }
     };
     auto publish = [&](int c0) {
         const int cn = min(CH, count - c0);
 #pragma unroll
         for (int u = 0; u < kScanSlots; ++u)
-            if (u < cn * KP && src_off[u] >= 0) rows[dst_off[u]] = pre[u];
+            if (u < cn * KP && src_off[u] != -1) rows[dst_off[u]] = (p.act && src_off[u] >= 0) ? seq_silu(pre[u]) : pre[u];
         if (tid < cn) {
-            const float dt = seq_softplus(pre_dt + bias);
-            dts[tid] = dt;
-            dts[CH + tid] = expf(-rate * dt);
+            if (lin) {
+                dts[tid] = pre_dt;
+                dts[CH + tid] = pre_dec;
+            } else {
+                const float dt = seq_softplus(pre_dt + bias);
+                dts[tid] = dt;
+                dts[CH + tid] = expf(-rate * dt);
+            }
         }
     };
     fetch(0);
@@ -239,21 +260,17 @@ extern "C" int64_t zls_ssm_scan_workspace_bytes(int64_t n_seq, int64_t max_count
     return n_seq * n_seg * heads * (2 * n_state * vdim + 1) * (int64_t)sizeof(float);
 }
 
-extern "C" int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int64_t dt_col0, const float* dt_bias, const float* a_log,
-                            const float* d, float* state, int64_t heads, int64_t vdim, int64_t n_state, int64_t groups, const zls_batch_t* b,
-                            float* y, void* workspace, int64_t seg_len, zl_stream_t s) {
-    ZL_CHECK_ARG(xbc && proj && dt_bias && a_log && d && state && y && seq_batch_ok(b), ZL_EINVAL);
-    ZL_CHECK_ARG(heads > 0 && vdim > 0 && n_state > 0 && groups > 0 && heads % groups == 0 && heads <= 65535, ZL_ESHAPE);
-    ZL_CHECK_ARG(dt_col0 >= 0 && dt_col0 + heads <= ld && vdim <= 1024, ZL_ESHAPE);
+// sizes the thread layout for (heads, vdim, n_state) in p and launches the scan (whole portions, or long ones in segments)
+static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, const zls_batch_t* b, void* workspace, int64_t seg_len,
+                       zl_stream_t s) {
+    ZL_CHECK_ARG(heads > 0 && vdim > 0 && n_state > 0 && heads <= 65535 && vdim <= 1024, ZL_ESHAPE);
     // ngl lanes share a column: the smallest power of two that leaves a thread at most 32 states
     int64_t ngl = 1;
     while ((n_state + ngl - 1) / ngl > 32) ngl <<= 1;
     ZL_CHECK_ARG(ngl <= 64 && ngl * vdim <= 1024, ZL_ELIMIT);
     const int64_t npt = ((n_state + ngl - 1) / ngl + 3) / 4 * 4;
     const int64_t threads = (ngl * vdim + 63) / 64 * 64;
-    ScanP p;
-    p.xbc = xbc; p.proj = proj; p.dt_bias = dt_bias; p.a_log = a_log; p.d = d; p.state = state; p.y = y; p.ld = ld;
-    p.dt_col0 = (int)dt_col0; p.heads = (int)heads; p.vdim = (int)vdim; p.n_state = (int)n_state; p.groups = (int)groups;
+    p.heads = (int)heads; p.vdim = (int)vdim; p.n_state = (int)n_state;
     p.ngl = (int)ngl; p.npt = (int)npt;
     const int64_t row = vdim + 2 * n_state;
     const int64_t kp = (row + threads - 1) / threads;                  // register slots a staged token row takes per thread
@@ -293,6 +310,31 @@ extern "C" int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int
 #undef SCAN_ANY
 #undef SCAN
     return zl_launch_status();
+}
+
+extern "C" int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int64_t dt_col0, const float* dt_bias, const float* a_log,
+                            const float* d, float* state, int64_t heads, int64_t vdim, int64_t n_state, int64_t groups, const zls_batch_t* b,
+                            float* y, void* workspace, int64_t seg_len, zl_stream_t s) {
+    ZL_CHECK_ARG(xbc && proj && dt_bias && a_log && d && state && y && seq_batch_ok(b), ZL_EINVAL);
+    ZL_CHECK_ARG(heads > 0 && groups > 0 && heads % groups == 0, ZL_ESHAPE);
+    ZL_CHECK_ARG(dt_col0 >= 0 && dt_col0 + heads <= ld, ZL_ESHAPE);
+    ScanP p = {};
+    p.xbc = xbc; p.proj = proj; p.dt_bias = dt_bias; p.a_log = a_log; p.d = d; p.state = state; p.y = y; p.ld = ld;
+    p.dt_col0 = (int)dt_col0; p.groups = (int)groups;
+    return launch_scan(p, heads, vdim, n_state, b, workspace, seg_len, s);
+}
+
+extern "C" int zls_decay_scan(const float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int act, const float* decay_h,
+                              const float* decay_t, const float* gain_t, int norm_col, float* state, int64_t heads, int64_t dim, int64_t vdim,
+                              const zls_batch_t* b, float* y, void* workspace, int64_t seg_len, zl_stream_t s) {
+    ZL_CHECK_ARG(proj && (decay_h || decay_t) && state && y && seq_batch_ok(b) && heads > 0 && dim > 0 && vdim > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ld && k_col0 >= 0 && k_col0 + heads * dim <= ld && v_col0 >= 0 &&
+                 v_col0 + heads * vdim <= ld && ld * kScanSlots < (1LL << 31), ZL_ESHAPE);
+    ScanP p = {};
+    p.proj = proj; p.state = state; p.y = y; p.ld = ld; p.groups = (int)heads;
+    p.kind = 1; p.act = act ? 1 : 0; p.ones = norm_col ? 1 : 0; p.q_col0 = (int)q_col0; p.k_col0 = (int)k_col0; p.v_col0 = (int)v_col0;
+    p.decay_h = decay_h; p.decay_t = decay_t; p.gain_t = gain_t;
+    return launch_scan(p, heads, vdim + p.ones, dim, b, workspace, seg_len, s);
 }
 
 extern "C" int zls_gated_group_norm(const float* y, const float* proj, int64_t ld, int64_t z_col0, const float* weight, float eps, int64_t rows,

@@ -1,5 +1,5 @@
 """Sequence mixers and feed-forwards for ragged steps: each is a weight container + the kernel sequence of its forward, with every
-constant a constructor argument, so that a model description picks and sizes them (tupitar.py does; another design can).
+constant a constructor argument, so that a model description picks and sizes them (tupitar.py and retotar.py do; another design can).
 
 A mixer's forward takes h (n_tok, width) in the serving format and the step's RaggedBatch and returns fp32 (n_tok, width).  What it keeps
 between steps it registers with the CacheManager in `bind`: per-token rows as a paged plane, per-sequence state as a slot state.
@@ -176,3 +176,241 @@ class PolyNormFF:
     def forward(self, h):
         z = seqops.gemm_nt(h, self.w_up)
         return seqops.gemm_nt(seqops.polynorm(z, self.coef, self.eps, h.dtype), self.w_down)
+
+
+def rotary_frequencies(n_rot, base, divide=1.0, device="cpu"):
+    """base^(-2i / n_rot) / divide for the n_rot / 2 pairs, worked out in float64 and rounded once to fp32"""
+    i = torch.arange(n_rot // 2, dtype=torch.float64)
+    return (torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / n_rot) / float(divide)).to(torch.float32).to(device)
+
+
+class WindowAttention:
+    """Softmax attention with grouped key / value heads over a paged cache: rotary positions on the first `rot_dims` coordinates of every
+    query and key head (pairs i, i + rot_dims / 2; every frequency divided by `rot_scaling`), queries and keys divided by their root mean
+    square afterwards (qk_norm), a sliding window of `window` positions (0: none), optionally
+      * values turned by their own position over all vdim coordinates before they are cached and the heads' sums turned back by the query's
+        position (rotate_values; frequencies from the same base, never scaled),
+      * the heads' softmax weights mixed by a (heads, heads) matrix after the softmax (tensor `talk`),
+      * a sigmoid gate per output coordinate computed from the mixer's input (tensor `g`),
+      * keys and values borrowed from another layer's cache (kv_source: that layer's WindowAttention; then no k / v tensors).
+    Tensors under `prefix`: q (heads*dim, width), k (kv_heads*dim, width), v (kv_heads*vdim, width), talk (heads, heads), g (heads*vdim, width),
+    o (width, heads*vdim).  q | k | v | g are one product."""
+
+    def __init__(self, name, width, heads, kv_heads, dim, vdim, scale, window, rot_dims, rot_base, rot_scaling, eps, qk_norm=True,
+                 rotate_values=True, talk=True, gate=True, kv_source=None):
+        if heads % kv_heads or rot_dims % 2 or rot_dims > dim or (rotate_values and vdim % 2):
+            raise ZLError("attention: heads must divide by kv_heads, rotated sizes must be even and fit the head")
+        if kv_source is not None and (kv_source.kv_heads, kv_source.dim, kv_source.vdim) != (kv_heads, dim, vdim):
+            raise ZLError("attention: a borrowed cache must have this layer's key / value shape")
+        self.name, self.width, self.heads, self.kv_heads, self.dim, self.vdim = name, width, heads, kv_heads, dim, vdim
+        self.scale, self.window, self.rot_dims, self.rot_base, self.rot_scaling = float(scale), int(window), rot_dims, float(rot_base), float(rot_scaling)
+        self.eps, self.qk_norm, self.rotate_values, self.has_talk, self.has_gate = float(eps), qk_norm, rotate_values, talk, gate
+        self.kv_source = kv_source
+        self.k_cache = self.v_cache = None
+
+    def _cols(self):
+        H, G, d, v = self.heads, self.kv_heads, self.dim, self.vdim
+        own = self.kv_source is None
+        kq, vq = H * d, H * d + (G * d if own else 0)
+        g0 = vq + (G * v if own else 0)
+        return kq, vq, g0, g0 + (H * v if self.has_gate else 0)
+
+    def _tables(self, device):
+        self.qk_freq = rotary_frequencies(self.rot_dims, self.rot_base, self.rot_scaling, device) if self.rot_dims else None
+        self.v_freq = rotary_frequencies(self.vdim, self.rot_base, 1.0, device) if self.rotate_values else None
+
+    def load(self, get, prefix, dtype, device):
+        H, G, d, v, W = self.heads, self.kv_heads, self.dim, self.vdim, self.width
+        parts = [_mat(get, prefix + "q", (H * d, W), dtype, device)]
+        if self.kv_source is None:
+            parts += [_mat(get, prefix + "k", (G * d, W), dtype, device), _mat(get, prefix + "v", (G * v, W), dtype, device)]
+        if self.has_gate:
+            parts.append(_mat(get, prefix + "g", (H * v, W), dtype, device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.talk = _mat(get, prefix + "talk", (H, H), torch.float32, device) if self.has_talk else None
+        self.w_o = _mat(get, prefix + "o", (W, H * v), dtype, device)
+        self._tables(device)
+        return self
+
+    def init_random(self, gen, dtype, device):
+        H, v, W = self.heads, self.vdim, self.width
+        self.w_in = _rand(gen, (self._cols()[3], W), W ** -0.5, dtype, device)
+        self.talk = (torch.eye(H, device=device) + 0.1 * torch.randn(H, H, generator=gen, device=device)) if self.has_talk else None
+        self.w_o = _rand(gen, (W, H * v), (H * v) ** -0.5, dtype, device)
+        self._tables(device)
+        return self
+
+    def bind(self, cache, dtype):
+        if self.kv_source is not None:                      # (the lender is an earlier layer: it is bound already)
+            self.k_cache, self.v_cache = self.kv_source.k_cache, self.kv_source.v_cache
+            return
+        self.k_cache = cache.add_plane(self.name + ".k", (self.kv_heads * self.dim,), dtype)
+        self.v_cache = cache.add_plane(self.name + ".v", (self.kv_heads * self.vdim,), dtype)
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.w_in, self.w_o))
+
+    def forward(self, h, batch):
+        H, G, d, v = self.heads, self.kv_heads, self.dim, self.vdim
+        k0, v0, g0, _ = self._cols()
+        own = self.kv_source is None
+        proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | k | v | gate]
+        seqops.rope_norm_store(proj, 0, k0, v0, H, G, d, v, self.qk_freq, self.rot_dims, self.v_freq, self.eps, self.qk_norm, batch,
+                               self.k_cache if own else None, self.v_cache if own else None)
+        acc = seqops.window_attention(proj, 0, self.k_cache, self.v_cache, batch, self.scale, self.window, H, G, d, v, all_kv=self.has_talk)
+        a = seqops.head_mix_gate(acc, self.talk, self.v_freq, proj if self.has_gate else None, g0, batch, H, G, v, h.dtype)
+        return seqops.gemm_nt(a, self.w_o)
+
+
+class DecayLinearAttention:
+    """Linear attention with a fixed decay per head: q, k, v = act(projections); S_t = decay_h S_{t-1} + k_t v_t^T, o_t = S_t^T q_t per head,
+    the state fp32 per sequence; then the RMS norm over all heads together with a weight, the sigmoid gate, the output projection.
+    Tensors under `prefix`: q, k (heads*dim, width), v, g (heads*vdim, width), norm (heads*vdim), o (width, heads*vdim)."""
+
+    def __init__(self, name, width, heads, dim, vdim, decay, eps, act="silu", norm_groups=1):
+        if len(decay) != heads:
+            raise ZLError("linear attention: one decay per head")
+        self.name, self.width, self.heads, self.dim, self.vdim = name, width, heads, dim, vdim
+        self.decay_values, self.eps, self.act, self.norm_groups = [float(x) for x in decay], float(eps), act, norm_groups
+        self.scan_segment = None
+
+    def load(self, get, prefix, dtype, device):
+        H, d, v, W = self.heads, self.dim, self.vdim, self.width
+        self.w_in = torch.cat([_mat(get, prefix + "q", (H * d, W), dtype, device), _mat(get, prefix + "k", (H * d, W), dtype, device),
+                               _mat(get, prefix + "v", (H * v, W), dtype, device), _mat(get, prefix + "g", (H * v, W), dtype, device)], dim=0).contiguous()
+        self.norm_w = _vec(get, prefix + "norm", H * v, device)
+        self.w_o = _mat(get, prefix + "o", (W, H * v), dtype, device)
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float64).to(torch.float32).to(device)
+        return self
+
+    def init_random(self, gen, dtype, device):
+        H, d, v, W = self.heads, self.dim, self.vdim, self.width
+        self.w_in = _rand(gen, (2 * H * d + 2 * H * v, W), W ** -0.5, dtype, device)
+        self.norm_w = torch.ones(H * v, device=device)
+        self.w_o = _rand(gen, (W, H * v), (H * v) ** -0.5, dtype, device)
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=device)
+        return self
+
+    def bind(self, cache, dtype):
+        self.state = cache.add_state(self.name + ".S", (self.heads, self.dim, self.vdim))
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.w_in, self.w_o))
+
+    def forward(self, h, batch):
+        H, d, v = self.heads, self.dim, self.vdim
+        proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | k | v | gate]
+        y = seqops.decay_scan(proj, 0, H * d, 2 * H * d, self.act == "silu", self.decay, None, None, False, self.state, H, d, v, batch,
+                              seg_len=self.scan_segment)
+        a = seqops.linear_attn_finish(y, False, 1.0, None, 0.0, H, v, self.norm_groups, self.norm_w, self.eps, proj, 2 * H * d + H * v, h.dtype)
+        return seqops.gemm_nt(a, self.w_o)
+
+
+class MLSTMMixer:
+    """Matrix memory with exponential gates (mLSTM): per head a log input gate i and a log forget gate f = log sigmoid(.), both capped by
+    cap * tanh(. / cap), a running maximum m (from 0) that keeps the exponentials in range:
+        m_t = max(f + m_{t-1}, i);  S_t = e^{f + m_{t-1} - m_t} S_{t-1} + e^{i - m_t} k v^T;  n_t the same with k alone
+        o = S_t^T q / (max(|n_t . q|, e^{-m_t}) + 1e-6),  q scaled by dim^-1/2
+    then each head divided by its root mean square, a weight over all heads, the sigmoid gate, the output projection.  S, n, m are fp32 per
+    sequence; n rides in the scan as one more value column that is 1 for every token.
+    Tensors under `prefix`: q, k (heads*dim, width), v, g (heads*vdim, width), i, f (heads, width), i.b, f.b (heads), norm (heads*vdim),
+    o (width, heads*vdim)."""
+
+    def __init__(self, name, width, heads, dim, vdim, gate_cap, eps, den_eps=1e-6):
+        self.name, self.width, self.heads, self.dim, self.vdim = name, width, heads, dim, vdim
+        self.cap, self.eps, self.den_eps = float(gate_cap), float(eps), float(den_eps)
+        self.scan_segment = None
+
+    def load(self, get, prefix, dtype, device):
+        H, d, v, W = self.heads, self.dim, self.vdim, self.width
+        self.w_in = torch.cat([_mat(get, prefix + "q", (H * d, W), dtype, device), _mat(get, prefix + "k", (H * d, W), dtype, device),
+                               _mat(get, prefix + "v", (H * v, W), dtype, device), _mat(get, prefix + "g", (H * v, W), dtype, device),
+                               _mat(get, prefix + "i", (H, W), dtype, device), _mat(get, prefix + "f", (H, W), dtype, device)], dim=0).contiguous()
+        self.i_bias, self.f_bias = _vec(get, prefix + "i.b", H, device), _vec(get, prefix + "f.b", H, device)
+        self.norm_w = _vec(get, prefix + "norm", H * v, device)
+        self.w_o = _mat(get, prefix + "o", (W, H * v), dtype, device)
+        return self
+
+    def init_random(self, gen, dtype, device):
+        H, d, v, W = self.heads, self.dim, self.vdim, self.width
+        self.w_in = _rand(gen, (2 * H * d + 2 * H * v + 2 * H, W), W ** -0.5, dtype, device)
+        self.i_bias = torch.zeros(H, device=device)
+        self.f_bias = torch.full((H,), 3.0, device=device)
+        self.norm_w = torch.ones(H * v, device=device)
+        self.w_o = _rand(gen, (W, H * v), (H * v) ** -0.5, dtype, device)
+        return self
+
+    def bind(self, cache, dtype):
+        self.state = cache.add_state(self.name + ".S", (self.heads, self.dim, self.vdim + 1))
+        self.m_state = cache.add_state(self.name + ".m", (self.heads,))
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.w_in, self.w_o))
+
+    def forward(self, h, batch):
+        H, d, v = self.heads, self.dim, self.vdim
+        proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | k | v | gate | i | f]
+        g0 = 2 * H * d + H * v
+        decay, gain, m = seqops.exp_gates(proj, g0 + H * v, g0 + H * v + H, self.i_bias, self.f_bias, self.cap, self.m_state, H, batch)
+        y = seqops.decay_scan(proj, 0, H * d, 2 * H * d, False, None, decay, gain, True, self.state, H, d, v, batch, seg_len=self.scan_segment)
+        a = seqops.linear_attn_finish(y, True, d ** -0.5, m, self.den_eps, H, v, H, self.norm_w, self.eps, proj, g0, h.dtype)
+        return seqops.gemm_nt(a, self.w_o)
+
+
+class RoutedExpertsFF:
+    """Mixture of gated feed-forward experts, down(silu(gate h) * (up h)), without biases.  The router gives one logit per expert and per
+    IDENTITY output (the last `identity` of its outputs: their "expert" returns h itself); probabilities = softmax over all outputs; an
+    output is chosen by probability + `correction`, within the `keep` best of `groups` equal groups of neighbouring outputs (a group scores
+    by its best member); the `top` chosen outputs are weighted by their plain probabilities (renormalised only if `renorm`).
+    Tensors under `prefix`: router (experts + identity, width), correction (experts + identity), e<j>.gate / e<j>.up (ff, width),
+    e<j>.down (width, ff).  Gate and up rows of all experts are stacked in blocks of 16 (16 gate rows, their 16 up rows), so that the grouped
+    product's epilogue finishes the activation."""
+
+    def __init__(self, width, ff, experts, top, identity=0, groups=1, keep=1, correction=True, renorm=False):
+        total = experts + identity
+        if groups < 1 or total % groups or not 1 <= keep <= groups or top > keep * (total // groups):
+            raise ZLError("experts: groups must divide the router outputs, and the kept groups must hold `top` outputs")
+        self.width, self.ff, self.experts, self.top, self.identity = width, ff, experts, top, identity
+        self.groups, self.keep, self.has_correction, self.renorm = groups, keep, correction, renorm
+        self.fused_act = ff % 16 == 0
+
+    def _pack_gate_up(self, gate, up):
+        if not self.fused_act:
+            return torch.cat([gate, up], dim=0)
+        f, w = gate.shape
+        return torch.stack([gate.reshape(f // 16, 16, w), up.reshape(f // 16, 16, w)], dim=1).reshape(2 * f, w)
+
+    def load(self, get, prefix, dtype, device):
+        E, f, W = self.experts, self.ff, self.width
+        self.w_router = _mat(get, prefix + "router", (E + self.identity, W), dtype, device)
+        self.correction = _vec(get, prefix + "correction", E + self.identity, device) if self.has_correction else None
+        self.w_gu = torch.empty((E, 2 * f, W), dtype=dtype, device=device)
+        self.w_down = torch.empty((E, W, f), dtype=dtype, device=device)
+        for e in range(E):
+            p = f"{prefix}e{e}."
+            self.w_gu[e] = self._pack_gate_up(_mat(get, p + "gate", (f, W), dtype, device), _mat(get, p + "up", (f, W), dtype, device))
+            self.w_down[e] = _mat(get, p + "down", (W, f), dtype, device)
+        return self
+
+    def init_random(self, gen, dtype, device):
+        E, f, W = self.experts, self.ff, self.width
+        self.w_router = _rand(gen, (E + self.identity, W), W ** -0.5, dtype, device)
+        self.correction = torch.zeros(E + self.identity, device=device) if self.has_correction else None
+        self.w_gu = _rand(gen, (E, 2 * f, W), W ** -0.5, dtype, device)
+        self.w_down = _rand(gen, (E, W, f), f ** -0.5, dtype, device)
+        return self
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.w_router, self.w_gu, self.w_down))
+
+    def forward(self, h):
+        logits = seqops.gemm_nt(h, self.w_router)                                 # fp32 sums of the products
+        ids, weights = seqops.moe_route(logits, self.correction, self.groups, self.keep, self.top, self.renorm)
+        sorted_tok, slot_pos, tiles, max_tiles = seqops.moe_align(ids, self.experts)
+        n_slots = ids.numel()
+        if self.fused_act:
+            a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype)
+        else:
+            a = seqops.silu_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots), h.dtype)
+        y = seqops.gemm_nt_grouped(a, None, self.w_down, tiles, max_tiles, n_slots)
+        return seqops.moe_combine(y, slot_pos, ids, weights, h, self.experts)

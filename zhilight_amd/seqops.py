@@ -16,7 +16,10 @@ BF16, F32 = 1, 2
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "libzhilight_amd_seq.so")
 SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_add_scalar_norm", "zls_scalar_norm_rows", "zls_polynorm",
-           "zls_latent_store", "zls_latent_attention", "zls_latent_attention_workspace_bytes", "zls_latent_attention_prompt", "zls_gemm_nt_gather", "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_ssm_scan_workspace_bytes", "zls_gated_group_norm"]
+           "zls_latent_store", "zls_latent_attention", "zls_latent_attention_workspace_bytes", "zls_latent_attention_prompt", "zls_gemm_nt_gather",
+           "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_ssm_scan_workspace_bytes", "zls_gated_group_norm", "zls_layer_norm",
+           "zls_add_layer_norm", "zls_rope_norm_store", "zls_window_attention", "zls_head_mix_gate", "zls_decay_scan", "zls_exp_gates",
+           "zls_linear_attn_finish", "zls_moe_route", "zls_moe_align", "zls_gemm_nt_grouped", "zls_silu_mul", "zls_moe_combine"]
 _STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
            -4: "exceeds a hardware limit"}
 
@@ -303,4 +306,180 @@ def gated_group_norm(y, proj, z_col0, weight, eps, norm_groups, dtype):
     out = torch.empty(y.shape, dtype=dtype, device=y.device)
     check(lib().zls_gated_group_norm(_p(y), _p(proj), _i(proj.shape[1]), _i(z_col0), _p(weight), _f(eps), _i(y.shape[0]), _i(y.shape[1]),
                                      _i(norm_groups), _p(out), C.c_int(dt_code(dtype)), _stream()), "gated_group_norm")
+    return out
+
+
+# ---- layer norm ------------------------------------------------------------------------------------------------------------------------
+def layer_norm(x, weight, bias, eps, dtype, rows=None):
+    """(x - mean) / sqrt(var + eps) * weight + bias of the rows `rows` (int32 device; None: all) of fp32 x, in `dtype`"""
+    _cuda(x, weight, bias, rows)
+    _f32(x, weight, bias)
+    if rows is not None and rows.dtype != torch.int32:
+        raise ZLError("layer_norm: rows must be int32")
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty((n, x.shape[1]), dtype=dtype, device=x.device)
+    check(lib().zls_layer_norm(_p(x), _p(rows), _p(weight), _p(bias), _f(eps), _i(n), _i(x.shape[1]), _p(out), C.c_int(dt_code(dtype)), _stream()),
+          "layer_norm")
+    return out
+
+
+def add_layer_norm(x, y, weight, bias, eps, next_weight=None, next_bias=None, dtype=None):
+    """x += layer_norm(y) in place; with next_weight also returns layer_norm(new x; next_weight, next_bias) in `dtype`"""
+    _cuda(x, y, weight, bias, next_weight, next_bias)
+    _f32(x, y, weight, bias, next_weight, next_bias)
+    if x.shape != y.shape or weight.numel() != x.shape[1]:
+        raise ZLError("add_layer_norm: shape mismatch")
+    h2 = torch.empty(x.shape, dtype=dtype, device=x.device) if next_weight is not None else None
+    check(lib().zls_add_layer_norm(_p(x), _p(y), _p(weight), _p(bias), _f(eps), _i(x.shape[0]), _i(x.shape[1]), _p(next_weight), _p(next_bias),
+                                   _p(h2), C.c_int(dt_code(dtype) if h2 is not None else BF16), _stream()), "add_layer_norm")
+    return h2
+
+
+# ---- softmax attention over paged keys and values -------------------------------------------------------------------------------------------
+def rope_norm_store(proj, q_col0, k_col0, v_col0, heads, kv_heads, dim, vdim, qk_freq, rot_dims, v_freq, eps, qk_norm, batch, k_cache, v_cache):
+    """rotate / norm the queries in place in proj; rotate / norm the keys and turn the values into the paged planes (None: queries only)"""
+    _cuda(proj, qk_freq, v_freq, k_cache, v_cache)
+    _f32(proj, qk_freq, v_freq)
+    if (qk_freq is not None and qk_freq.numel() != rot_dims // 2) or (v_freq is not None and v_freq.numel() != vdim // 2):
+        raise ZLError("rope_norm_store: one frequency per rotated pair")
+    if k_cache is not None:
+        if tuple(k_cache.shape[1:]) != (batch.c.page_size, kv_heads * dim) or tuple(v_cache.shape[1:]) != (batch.c.page_size, kv_heads * vdim) \
+                or k_cache.dtype != v_cache.dtype:
+            raise ZLError("rope_norm_store: planes must be (pages, page_size, kv_heads * dim | vdim)")
+    code = dt_code(k_cache.dtype) if k_cache is not None else F32
+    check(lib().zls_rope_norm_store(_p(proj), _i(proj.shape[1]), _i(q_col0), _i(k_col0), _i(v_col0), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
+                                    _p(qk_freq), _i(rot_dims), _p(v_freq), _f(eps), C.c_int(int(qk_norm)), batch.ref, _p(k_cache), _p(v_cache),
+                                    C.c_int(code), _stream()), "rope_norm_store")
+
+
+def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, kv_heads, dim, vdim, all_kv):
+    """fp32 (n_tok, heads, [kv_heads,] vdim): every query head's softmax weights applied to its own (all_kv False) or every kv head's values"""
+    _cuda(q, k_cache, v_cache)
+    _f32(q)
+    if tuple(k_cache.shape[1:]) != (batch.c.page_size, kv_heads * dim) or tuple(v_cache.shape[1:]) != (batch.c.page_size, kv_heads * vdim):
+        raise ZLError("window_attention: planes must be (pages, page_size, kv_heads * dim | vdim)")
+    acc = torch.empty((batch.n_tok, heads, kv_heads if all_kv else 1, vdim), dtype=torch.float32, device=q.device)
+    check(lib().zls_window_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _f(scale), _i(window), _i(heads),
+                                     _i(kv_heads), _i(dim), _i(vdim), C.c_int(int(all_kv)), _p(acc), C.c_int(dt_code(k_cache.dtype)), _stream()),
+          "window_attention")
+    return acc
+
+
+def head_mix_gate(acc, talk, v_freq, gate, g_col0, batch, heads, kv_heads, vdim, dtype):
+    _cuda(acc, talk, v_freq, gate)
+    _f32(acc, talk, v_freq, gate)
+    if talk is not None and tuple(talk.shape) != (heads, heads):
+        raise ZLError("head_mix_gate: the mixing matrix is (heads, heads)")
+    if acc.numel() != batch.n_tok * heads * (kv_heads if talk is not None else 1) * vdim:
+        raise ZLError("head_mix_gate: acc does not fit")
+    out = torch.empty((batch.n_tok, heads * vdim), dtype=dtype, device=acc.device)
+    check(lib().zls_head_mix_gate(_p(acc), _p(talk), _p(v_freq), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), batch.ref,
+                                  _i(heads), _i(kv_heads), _i(vdim), _p(out), C.c_int(dt_code(dtype)), _stream()), "head_mix_gate")
+    return out
+
+
+# ---- linear attention with a scalar decay -----------------------------------------------------------------------------------------------------
+def decay_scan(proj, q_col0, k_col0, v_col0, act, decay_h, decay_t, gain_t, norm_col, state, heads, dim, vdim, batch, seg_len=None):
+    """S <- a S + b k v^T, y = S^T q per head over the step's portions; fp32 y (n_tok, heads * (vdim + norm_col))"""
+    _cuda(proj, decay_h, decay_t, gain_t, state)
+    _f32(proj, decay_h, decay_t, gain_t, state)
+    P = vdim + (1 if norm_col else 0)
+    if tuple(state.shape[1:]) != (heads, dim, P):
+        raise ZLError("decay_scan: state must be (slots, heads, dim, vdim + norm_col)")
+    for t in (decay_t, gain_t):
+        if t is not None and tuple(t.shape) != (batch.n_tok, heads):
+            raise ZLError("decay_scan: per-token decays / gains are (n_tok, heads)")
+    y = torch.empty((batch.n_tok, heads * P), dtype=torch.float32, device=proj.device)
+    seg_len = SCAN_SEGMENT if seg_len is None else seg_len
+    ws = None
+    if seg_len > 0 and batch.c.max_count > seg_len:
+        ws = torch.empty(int(lib().zls_ssm_scan_workspace_bytes(_i(batch.n_seq), _i(batch.c.max_count), _i(seg_len), _i(heads), _i(P), _i(dim))) // 4,
+                         dtype=torch.float32, device=proj.device)
+    check(lib().zls_decay_scan(_p(proj), _i(proj.shape[1]), _i(q_col0), _i(k_col0), _i(v_col0), C.c_int(int(act)), _p(decay_h), _p(decay_t),
+                               _p(gain_t), C.c_int(int(norm_col)), _p(state), _i(heads), _i(dim), _i(vdim), batch.ref, _p(y), _p(ws), _i(seg_len),
+                               _stream()), "decay_scan")
+    return y
+
+
+def exp_gates(proj, i_col0, f_col0, i_bias, f_bias, cap, m_state, heads, batch):
+    """capped exponential gates with a running maximum: (decay, gain, m) fp32 (n_tok, heads) each; m_state (slots, heads) moves on"""
+    _cuda(proj, i_bias, f_bias, m_state)
+    _f32(proj, i_bias, f_bias, m_state)
+    out = torch.empty((3, batch.n_tok, heads), dtype=torch.float32, device=proj.device)
+    check(lib().zls_exp_gates(_p(proj), _i(proj.shape[1]), _i(i_col0), _i(f_col0), _p(i_bias), _p(f_bias), _f(cap), _p(m_state), _i(heads),
+                              batch.ref, _p(out[0]), _p(out[1]), _p(out[2]), _stream()), "exp_gates")
+    return out[0], out[1], out[2]
+
+
+def linear_attn_finish(y, norm_col, q_scale, m_vals, den_eps, heads, vdim, norm_groups, weight, eps, gate, g_col0, dtype):
+    _cuda(y, m_vals, weight, gate)
+    _f32(y, m_vals, weight, gate)
+    n_tok = y.shape[0]
+    if y.shape[1] != heads * (vdim + (1 if norm_col else 0)):
+        raise ZLError("linear_attn_finish: y does not fit")
+    out = torch.empty((n_tok, heads * vdim), dtype=dtype, device=y.device)
+    check(lib().zls_linear_attn_finish(_p(y), _i(int(norm_col)), _f(q_scale), _p(m_vals), _f(den_eps), _i(heads), _i(vdim), _i(norm_groups),
+                                       _p(weight), _f(eps), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), _i(n_tok), _p(out),
+                                       C.c_int(dt_code(dtype)), _stream()), "linear_attn_finish")
+    return out
+
+
+# ---- mixture of experts ------------------------------------------------------------------------------------------------------------------
+MOE_TILE = 64
+
+
+def moe_route(logits, correction, groups, keep, top, renorm=False):
+    _cuda(logits, correction)
+    _f32(logits, correction)
+    n_tok, n_out = logits.shape
+    if correction is not None and correction.numel() != n_out:
+        raise ZLError("moe_route: one correction per router output")
+    ids = torch.empty((n_tok, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((n_tok, top), dtype=torch.float32, device=logits.device)
+    check(lib().zls_moe_route(_p(logits), _i(n_tok), _i(n_out), _p(correction), _i(groups), _i(keep), _i(top), C.c_int(int(renorm)), _p(ids),
+                              _p(weights), _stream()), "moe_route")
+    return ids, weights
+
+
+def moe_align(ids, n_experts):
+    """(sorted_tok, slot_pos, tiles, max_tiles) of the (token, choice) pairs sorted by expert"""
+    _cuda(ids)
+    n_tok, top = ids.shape
+    n_slots = n_tok * top
+    max_tiles = n_slots // MOE_TILE + n_experts
+    buf = torch.empty(2 * n_slots + 3 * max_tiles, dtype=torch.int32, device=ids.device)
+    sorted_tok, slot_pos, tiles = buf[:n_slots], buf[n_slots:2 * n_slots], buf[2 * n_slots:]
+    check(lib().zls_moe_align(_p(ids), _i(n_slots), _i(top), _i(n_experts), _i(MOE_TILE), _p(sorted_tok), _p(slot_pos), _p(tiles), _i(max_tiles),
+                              _stream()), "moe_align")
+    return sorted_tok, slot_pos, tiles, max_tiles
+
+
+def gemm_nt_grouped(x, x_rows, w, tiles, max_tiles, n_rows, gated=False, out_dtype=torch.float32):
+    """rows of x (gathered by x_rows, or in sorted order) times their expert's block of w (experts, n, k); (n_rows, n or n / 2 gated)"""
+    _cuda(x, x_rows, w, tiles)
+    E, n, k = w.shape
+    if x.shape[1] != k or x.dtype != w.dtype:
+        raise ZLError("gemm_nt_grouped: size K / dtype mismatch")
+    out = torch.empty((n_rows, n // 2 if gated else n), dtype=out_dtype, device=x.device)
+    check(lib().zls_gemm_nt_grouped(_p(x), _i(x.stride(0)), _p(x_rows), _p(w), _p(tiles), _i(max_tiles), _p(out), _i(out.shape[1]), _i(n), _i(k),
+                                    C.c_int(int(gated)), C.c_int(dt_code(x.dtype)), C.c_int(dt_code(out_dtype)), _stream()), "gemm_nt_grouped")
+    return out
+
+
+def silu_mul(gu, dtype):
+    _cuda(gu)
+    _f32(gu)
+    rows, two_ff = gu.shape
+    out = torch.empty((rows, two_ff // 2), dtype=dtype, device=gu.device)
+    check(lib().zls_silu_mul(_p(gu), _i(rows), _i(two_ff // 2), _p(out), C.c_int(dt_code(dtype)), _stream()), "silu_mul")
+    return out
+
+
+def moe_combine(y, slot_pos, ids, weights, h, n_experts):
+    _cuda(y, slot_pos, ids, weights, h)
+    _f32(y, weights)
+    n_tok, top = ids.shape
+    out = torch.empty((n_tok, h.shape[1]), dtype=torch.float32, device=h.device)
+    check(lib().zls_moe_combine(_p(y), _p(slot_pos), _p(ids), _p(weights), _p(h), _i(n_tok), _i(top), _i(n_experts), _i(h.shape[1]), _p(out),
+                                C.c_int(dt_code(h.dtype)), _stream()), "moe_combine")
     return out
