@@ -171,14 +171,20 @@ def moe_ff(h, sd, pfx, f):
 
 
 # ---- the model -------------------------------------------------------------------------------------------------------------------------
-def forward(cfg, sd, tokens, return_layers=False):
-    """logits (T, vocab) of one whole sequence; with return_layers also the residual stream after every layer"""
+def forward(cfg, sd, tokens, return_layers=False, bf16_inputs=False):
+    """logits (T, vocab) of one whole sequence; with return_layers also the residual stream after every layer.
+    bf16_inputs: every sub-layer's input (the norm before it) is rounded to bfloat16, as bf16 serving hands it to the matrix products --
+    the reference for sizes at which that rounding alone moves single positions by much (a denominator near its floor)."""
     eps = cfg["norm"]["eps"]
+
+    def pre(u, name):
+        h = layer_norm(u, sd, name, eps)
+        return h.to(torch.bfloat16).to(F64) if bf16_inputs else h
     x = w64(sd, "embed")[torch.as_tensor(tokens, dtype=torch.long)] * cfg["embedding"]["scale"]
     kv, layers = {}, []
     for i, l in enumerate(cfg["layers"]):
         p, m = f"l{i}.", l["mixer"]
-        h = layer_norm(x, sd, p + "norm1", eps)
+        h = pre(x, p + "norm1")
         if l["type"] == "attention":
             if m.get("kv_from") is None:
                 kv[i] = attention_kv(h, sd, p + "mix.", m, eps)
@@ -193,8 +199,107 @@ def forward(cfg, sd, tokens, return_layers=False):
             raise ValueError(l["type"])
         x = x + layer_norm(y, sd, p + "norm1b", eps)
         if l.get("mlp") is not None:
-            y = moe_ff(layer_norm(x, sd, p + "norm2", eps), sd, p + "mlp.", l["mlp"])
+            y = moe_ff(pre(x, p + "norm2"), sd, p + "mlp.", l["mlp"])
             x = x + layer_norm(y, sd, p + "norm2b", eps)
         layers.append(x.clone())
-    logits = layer_norm(x, sd, "final.norm", eps) @ w64(sd, "head").T
+    logits = pre(x, "final.norm") @ w64(sd, "head").T
     return (logits, layers) if return_layers else logits
+
+
+# ---- small configurations and random weights for the tests --------------------------------------------------------------------------------
+SIZES = [
+    # attention: 2 query heads per kv head, a third of the head rotated; experts in 4 groups of 2 with 2 identity outputs
+    dict(att=dict(heads=4, kv_heads=2, dim=24, vdim=16, scale=0.7, mask={"size": 20}, rot={"dims": 8, "base": 10000.0, "scaling": {"factor": 4.0}}),
+         lin=dict(heads=3, dim=16, vdim=24, decay=[0.5, 0.9, 0.995]),
+         mls=dict(heads=2, dim=40, vdim=12, gate_cap=10.0),
+         moe=dict(ff=48, experts=6, identity=2, groups=4, keep=2, top=3)),
+    # one kv head per query head, the whole head rotated, no scaling, a window of 5; one group, no identity, one expert per token, an ff that
+    # is no multiple of 16
+    dict(att=dict(heads=3, kv_heads=3, dim=10, vdim=22, scale=0.3, mask={"size": 5}, rot={"dims": 10, "base": 100.0, "scaling": {"factor": 1.0}}),
+         lin=dict(heads=1, dim=8, vdim=8, decay=[0.97]),
+         mls=dict(heads=5, dim=6, vdim=20, gate_cap=4.0),
+         moe=dict(ff=40, experts=5, identity=0, groups=1, keep=1, top=1)),
+    # heads wider than a wave, one kv head for all, a window longer than the prompts; many experts, more identity outputs
+    dict(att=dict(heads=6, kv_heads=1, dim=72, vdim=80, scale=0.12, mask={"size": 4096}, rot={"dims": 36, "base": 500000.0, "scaling": {"factor": 1.5}}),
+         lin=dict(heads=2, dim=100, vdim=130, decay=[0.8, 0.999]),
+         mls=dict(heads=2, dim=72, vdim=36, gate_cap=30.0),
+         moe=dict(ff=32, experts=13, identity=3, groups=2, keep=1, top=4)),
+]
+_KIND = {"attention": "att", "shared": "att", "lightning": "lin", "mlstm": "mls"}
+
+
+def small_config(order=("lightning", "mlstm", "attention", "shared"), width=72, vocab=97, sizes=0, no_mlp_at=()):
+    """order: mixer types; "shared" = an attention layer on the keys and values of the nearest earlier attention layer with its own"""
+    z = SIZES[sizes]
+    layers, lender = [], None
+    for i, t in enumerate(order):
+        m = {k: (dict(v) if isinstance(v, dict) else v) for k, v in z[_KIND[t]].items()}
+        if t == "shared":
+            m["kv_from"] = lender
+        elif t == "attention":
+            lender = i
+        f = z["moe"]
+        mlp = None if i in no_mlp_at else {"kind": "moe", "expert": {"ff": f["ff"]}, "router": {
+            "experts": f["experts"], "identity": f["identity"], "top": f["top"], "groups": {"count": f["groups"], "keep": f["keep"]}}}
+        layers.append({"type": "attention" if t == "shared" else t, "mixer": m, "mlp": mlp})
+    return {"architecture": "Retotar", "embedding": {"scale": 0.7}, "layers": layers, "norm": {"eps": 1e-5}, "vocab": vocab, "width": width}
+
+
+def random_weights(cfg, seed=0, fixed_choice=False):
+    """every tensor the configuration asks for, bf16-representable values (so that both serving formats start from the same numbers).
+    fixed_choice: the routers' correction terms lie more than 1 apart, so that they alone order the choice scores (probabilities lie in
+    [0, 1]) and no choice is a close call; the weights of the chosen outputs still follow the probabilities."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    sd = {}
+
+    def mat(name, rows, cols, std=None):
+        sd[name] = (torch.randn(rows, cols, generator=g) * (std if std is not None else cols ** -0.5)).to(torch.bfloat16)
+
+    def norm(name, n):
+        sd[name] = (1.0 + 0.2 * torch.randn(n, generator=g)).to(torch.bfloat16)
+        sd[name + ".b"] = (0.1 * torch.randn(n, generator=g)).to(torch.bfloat16)
+
+    mat("embed", cfg["vocab"], W, 1.5)
+    mat("head", cfg["vocab"], W)
+    norm("final.norm", W)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        norm(p + "norm1", W)
+        norm(p + "norm1b", W)
+        H, d, v = m["heads"], m["dim"], m["vdim"]
+        mat(p + "mix.q", H * d, W)
+        mat(p + "mix.g", H * v, W)
+        mat(p + "mix.o", W, H * v)
+        if l["type"] == "attention":
+            if m.get("kv_from") is None:
+                mat(p + "mix.k", m["kv_heads"] * d, W)
+                mat(p + "mix.v", m["kv_heads"] * v, W)
+            sd[p + "mix.talk"] = (torch.eye(H) * 0.8 + 0.3 * torch.randn(H, H, generator=g)).to(torch.bfloat16)
+        else:
+            mat(p + "mix.k", H * d, W)
+            mat(p + "mix.v", H * v, W)
+            sd[p + "mix.norm"] = (1.0 + 0.2 * torch.randn(H * v, generator=g)).to(torch.bfloat16)
+            if l["type"] == "mlstm":
+                # keys lean towards the queries, so that the normaliser n . q seldom passes through zero: there the output is a quotient of
+                # two small numbers, and any rounding of the input moves it by much (the floor of the denominator has its own test)
+                sd[p + "mix.k"] = (0.8 * sd[p + "mix.q"].float() + 0.6 * sd[p + "mix.k"].float()).to(torch.bfloat16)
+                mat(p + "mix.i", H, W, 0.4)
+                mat(p + "mix.f", H, W, 0.4)
+                sd[p + "mix.i.b"] = (0.5 * torch.randn(H, generator=g)).to(torch.bfloat16)
+                sd[p + "mix.f.b"] = (2.0 + torch.randn(H, generator=g)).to(torch.bfloat16)
+        f = l.get("mlp")
+        if f is not None:
+            norm(p + "norm2", W)
+            norm(p + "norm2b", W)
+            r = f["router"]
+            total = r["experts"] + r.get("identity", 0)
+            mat(p + "mlp.router", total, W, 2.0 * W ** -0.5)
+            sd[p + "mlp.correction"] = (0.3 * torch.randn(total, generator=g) - 0.5).to(torch.bfloat16)      # choice scores go negative
+            if fixed_choice:
+                sd[p + "mlp.correction"] = (-1.5 * torch.randperm(total, generator=g).double()).to(torch.bfloat16)
+            for e in range(r["experts"]):
+                mat(f"{p}mlp.e{e}.gate", f["expert"]["ff"], W)
+                mat(f"{p}mlp.e{e}.up", f["expert"]["ff"], W)
+                mat(f"{p}mlp.e{e}.down", W, f["expert"]["ff"])
+    return sd
