@@ -17,9 +17,11 @@ fields, `roofline` (the W4A16 GEMV kernel: algorithmic bytes / HIP-event time, v
 `cpu_baseline` (the CPU oracle timed on a bounded sample on this box's host cores).
 
     python bench.py --mixers 1b,8b [--seq 2048]
+    python bench.py --retotar 1b,8b [--seq 2048]
 
 is a different measurement with its own JSON line: prefill / decode throughput of the ragged-step engine's latent-attention, state-space
-and hybrid stacks (zhilight_amd/tupitar.py) beside the dense bf16 Llama-shaped stack of equal width, 4 layers each, random weights.
+and hybrid stacks (zhilight_amd/tupitar.py) beside the dense bf16 Llama-shaped stack of equal width, 4 layers each, random weights;
+--retotar the same for the Retotar stacks (zhilight_amd/retotar.py) beside the Tupitar hybrid of equal width.
 """
 import argparse
 import json
@@ -517,8 +519,92 @@ def bench_sequence_mixers(args, dev):
                       "results": results}))
 
 
+RETOTAR_BENCH_SIZES = {
+    # name: width; attention heads / key-value heads x head size, window, rotated part; linear-attention heads x key size x value size; mLSTM the
+    #       same; experts x their ff, picks per token.  The picked experts' three matrices hold what SEQ_BENCH_SIZES' two-matrix ff of the
+    #       same name holds, so the Tupitar hybrid of equal width beside it moves the same feed-forward weights per token.
+    "1b": dict(width=2048, heads=16, kv_heads=4, dim=128, window=1024, rot=64, l_heads=16, l_dim=128, l_vdim=128, m_heads=8, m_dim=128,
+               m_vdim=128, experts=16, ff=1360, top=4, identity=2, groups=3, keep=2),
+    "8b": dict(width=4096, heads=32, kv_heads=8, dim=128, window=1024, rot=64, l_heads=32, l_dim=128, l_vdim=128, m_heads=16, m_dim=128,
+               m_vdim=128, experts=32, ff=2384, top=4, identity=4, groups=4, keep=2),
+}
+
+
+def bench_retotar(args, dev):
+    """--retotar: prefill and decode throughput of Retotar stacks (zhilight_amd/retotar.py: windowed attention with mixed heads, decayed
+    linear attention, mLSTM, routed experts) beside the closest existing model of equal width, the Tupitar hybrid of the ragged-step engine
+    (latent attention + state-space layers, PolyNorm feed-forward), 4 layers each, random weights, eager launches.  One JSON line."""
+    from zhilight_amd.engine import Engine, Entry
+    from zhilight_amd.retotar import RetotarConfig, RetotarLayerConfig, RetotarModel
+    from zhilight_amd.tupitar import TupitarConfig, TupitarLayerConfig, TupitarModel
+    seq, vocab, results = args.seq, 32000, []
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def measure(label, name, model):
+        toks = torch.randint(0, vocab, (seq,)).tolist()
+        for batch in (1, 8):
+            eng = Engine(model, max_tokens=batch * (seq + 64), max_seqs=batch)
+
+            def prefill():
+                eng.run_step([Entry("p", toks, [seq - 1])])
+                eng.release("p")
+            if batch == 1:
+                ms = timed(prefill, 3)
+                results.append(dict(model=label, size=name, phase="prefill", tokens=seq, ms=round(ms, 3), tokens_per_s=round(seq / ms * 1e3)))
+            for b in range(batch):
+                eng.run_step([Entry(f"d{b}", toks[:seq - 40], [])])
+
+            def decode():
+                eng.run_step([Entry(f"d{b}", [7], [0]) for b in range(batch)])
+            ms = timed(decode, 20)
+            results.append(dict(model=label, size=name, phase="decode", batch=batch, context=seq - 40, ms=round(ms, 3),
+                                tokens_per_s=round(batch / ms * 1e3)))
+            del eng
+
+    for name in args.retotar.split(","):
+        z = RETOTAR_BENCH_SIZES[name]
+        total = z["experts"] + z["identity"]
+        mlp = dict(kind="moe", expert=dict(ff=z["ff"]), router=dict(experts=z["experts"], identity=z["identity"], top=z["top"],
+                                                                    groups=dict(count=z["groups"] if total % z["groups"] == 0 else 1, keep=z["keep"])))
+        if mlp["router"]["groups"]["count"] == 1:
+            mlp["router"]["groups"]["keep"] = 1
+        att = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5, mask=dict(size=z["window"]),
+                   rot=dict(dims=z["rot"], base=1e6, scaling=dict(factor=1.0)))
+        lin = dict(heads=z["l_heads"], dim=z["l_dim"], vdim=z["l_vdim"], decay=[1.0 - 2.0 ** -(3 + 5 * h / z["l_heads"]) for h in range(z["l_heads"])])
+        mls = dict(heads=z["m_heads"], dim=z["m_dim"], vdim=z["m_vdim"], gate_cap=15.0)
+        A = lambda **kw: RetotarLayerConfig("attention", dict(att, **kw), mlp)
+        L, M = RetotarLayerConfig("lightning", lin, mlp), RetotarLayerConfig("mlstm", mls, mlp)
+        for label, layers in (("attention x4", [A(), A(kv_from=0), A(), A(kv_from=2)]), ("lightning x4", [L] * 4), ("mlstm x4", [M] * 4),
+                              ("hybrid (l, m, a, a')", [L, M, A(), A(kv_from=2)])):
+            model = RetotarModel(RetotarConfig(vocab, z["width"], 1.0, 1e-6, 1 << 24, layers), "bfloat16", dev).init_random(1)
+            measure("retotar " + label, name, model)
+            del model
+        t = SEQ_BENCH_SIZES[name]
+        tatt = TupitarLayerConfig("latent_attention", dict(heads=t["heads"], dim=t["dim"], vdim=t["dim"], kv_rank=t["rank"], scale=t["dim"] ** -0.5),
+                                  dict(ff=t["ff"], kind="dense"))
+        tssm = TupitarLayerConfig("mamba2", dict(heads=t["m_heads"], vdim=t["m_vdim"], state=t["state"], groups=t["groups"], conv=4,
+                                                 norm_groups=t["groups"]), dict(ff=t["ff"], kind="dense"))
+        model = TupitarModel(TupitarConfig(vocab, t["width"], seq + 64, 1.0, 1e-6, [tatt, tatt, tssm, tatt]), "bfloat16", dev).init_random(1)
+        measure("tupitar hybrid (a, a, m, a)", name, model)
+        del model
+    print(json.dumps({"metric": "retotar_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": 4, "results": results}))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--retotar", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of Retotar stacks beside the Tupitar hybrid of equal "
+                         "width; comma-separated sizes of " + ", ".join(RETOTAR_BENCH_SIZES))
     ap.add_argument("--mixers", default="", metavar="SIZES",
                     help="instead of the default workload: prefill / decode throughput of the ragged-step engine's latent-attention + "
                          "state-space model beside the dense Llama-shaped stack of equal width; comma-separated sizes of " + ", ".join(SEQ_BENCH_SIZES))
@@ -558,6 +644,8 @@ def main():
 
     if args.mixers:
         return bench_sequence_mixers(args, dev)
+    if args.retotar:
+        return bench_retotar(args, dev)
     from zhilight_amd import ops  # noqa: F401  (raises if the HIP library is missing)
     from zhilight_amd.llama import LLaMA, ModelConfig, QuantConfig
 

@@ -143,8 +143,8 @@ int zls_add_layer_norm(float* x, const float* y, const float* w, const float* b,
  *   i + rot_dims / 2 and the pair (u, v) becomes (u cos a - v sin a, v cos a + u sin a), a = p * qk_freq[i]; the other coordinates stay;
  *   with qk_norm != 0 every head is then divided by sqrt(mean(head^2) + eps);
  *   values (kv_heads x vdim from v_col0): with v_freq (nullable) turned the same way over ALL vdim coordinates, a = p * v_freq[i].
- * Queries are written back to proj; keys and values go to the token's row of k_cache (pages, page_size, kv_heads * dim) and v_cache
- * (pages, page_size, kv_heads * vdim) in `dtype`.  k_cache NULL (then v_cache too): only the queries are served -- a layer that reads
+ * Queries are written back to proj; keys go to the token's row of k_cache (pages, page_size, kv_heads * dim), values to the token's
+ * column of v_cache, whose pages are transposed: (pages, kv_heads * vdim, page_size); both in `dtype`.  k_cache NULL (then v_cache too): only the queries are served -- a layer that reads
  * another layer's cache.  qk_freq fp32 (rot_dims / 2; rot_dims even, <= dim; 0: no rotation), v_freq fp32 (vdim / 2; vdim even).
  * dim, vdim <= 512. */
 int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, int64_t heads, int64_t kv_heads, int64_t dim,
@@ -153,20 +153,33 @@ int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int64_t k_col0,
 
 /* Softmax attention of every token over the cached keys j of its sequence with 0 <= p - j < window (window <= 0: all j <= p):
  *   w_g(j) = softmax_j(scale * q_g . k_c(g)(j)),  c(g) = g / (heads / kv_heads)
- *   all_kv == 0:  acc[t][g][:]    = sum_j w_g(j) v_c(g)(j)                      acc fp32 (n_tok, heads, vdim)
- *   all_kv != 0:  acc[t][g][c][:] = sum_j w_g(j) v_c(j) for EVERY kv head c     acc fp32 (n_tok, heads, kv_heads, vdim)
+ *   all_kv == 0:  a[g][:]    = sum_j w_g(j) v_c(g)(j)                      nv = vdim numbers per head
+ *   all_kv != 0:  a[g][c][:] = sum_j w_g(j) v_c(j) for EVERY kv head c     nv = kv_heads * vdim
  * The second form is what mixing the heads' weights needs (zls_head_mix_gate): sum_j (sum_g T[h][g] w_g(j)) v_c(h)(j) =
- * sum_g T[h][g] acc[g][c(h)].  q fp32 (n_tok, ldq) from q_col0 (as zls_rope_norm_store left it).  Scores, weights and sums are fp32; keys of a
- * long context are walked in chunks with a running maximum.  (all_kv ? kv_heads : 1) * vdim <= 2048. */
+ * sum_g T[h][g] a[g][c(h)].  q fp32 (n_tok, ldq) from q_col0 (as zls_rope_norm_store left it).  Scores, weights and sums are fp32.
+ * The pages of a token's window are divided over n_splits workgroups (pages_per_split each, from the page of the window's oldest key;
+ * n_splits * pages_per_split must cover the longest window of the step); split s leaves acc[t][g][s][:] = sum_j e^(s_j - m) v_j,
+ * unnormalised, and ml[t][g][s] = (m, sum_j e^(s_j - m)); zls_head_mix_gate merges them.  acc fp32 (n_tok, heads, n_splits, nv), ml fp32
+ * (n_tok, heads, n_splits, 2).  single_only != 0: only sequences that bring ONE token are served (portions: zls_window_attention_prompt).
+ * The value plane holds a page TRANSPOSED, (kv_heads, vdim, page_size), as zls_rope_norm_store writes it.  nv <= 2048, page_size <= 128
+ * and a multiple of 8. */
 int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
                          float scale, int64_t window, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc,
-                         int dtype, zl_stream_t s);
+                         float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype, zl_stream_t s);
+/* The same attention for query TILES on the matrix cores, bf16 only: tile i = tiles[3 i ..] = (first flat token, rows <= 64, sequence
+ * index), consecutive tokens of one sequence.  Writes split 0 of acc for its tokens, already normalised, with ml = (0, 1), and
+ * ml = (-inf, 0) for the other splits.  page_size 64, dim % 8 == 0, dim <= 256, vdim % 16 == 0. */
+int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
+                                const int32_t* tiles, int64_t n_tiles, float scale, int64_t window, int64_t heads, int64_t kv_heads,
+                                int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits, int dtype, zl_stream_t s);
 
-/* out[t][h][:] = turn_back(sum_g talk[h][g] acc[t][g][c(h)][:]) * sigmoid(gate[t][h * vdim + :])
- * talk fp32 (heads, heads), NULL: no mixing, acc is (n_tok, heads, vdim); v_freq (nullable): pair (m, m + vdim / 2) is turned by
- * -p * v_freq[m]; gate fp32 (n_tok, ldg) from g_col0, NULL: no gate; out (n_tok, heads * vdim) in `dtype`. */
-int zls_head_mix_gate(const float* acc, const float* talk, const float* v_freq, const float* gate, int64_t ldg, int64_t g_col0,
-                      const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out, int dtype, zl_stream_t s);
+/* out[t][h][:] = turn_back(sum_g talk[h][g] a[t][g][c(h)][:]) * sigmoid(gate[t][h * vdim + :]), a = the splits of acc merged:
+ * a[t][g] = sum_s e^(m_s - M) acc[t][g][s] / sum_s e^(m_s - M) l_s.
+ * talk fp32 (heads, heads), NULL: no mixing, acc holds vdim numbers per head and split; v_freq (nullable): pair (m, m + vdim / 2) is turned
+ * by -p * v_freq[m]; gate fp32 (n_tok, ldg) from g_col0, NULL: no gate; out (n_tok, heads * vdim) in `dtype`. */
+int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_splits, const float* talk, const float* v_freq, const float* gate,
+                      int64_t ldg, int64_t g_col0, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out, int dtype,
+                      zl_stream_t s);
 
 /* ---- linear attention with a scalar decay per head and token ---------------------------------------------------------------------- */
 /* S_t = a_t S_{t-1} + b_t k_t v_t^T,  y_t = S_t^T q_t   per head, S fp32 (dim x vdim) carried in state[slot].

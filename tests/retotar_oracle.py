@@ -224,6 +224,11 @@ SIZES = [
          lin=dict(heads=2, dim=100, vdim=130, decay=[0.8, 0.999]),
          mls=dict(heads=2, dim=72, vdim=36, gate_cap=30.0),
          moe=dict(ff=32, experts=13, identity=3, groups=2, keep=1, top=4)),
+    # as many kv heads as query heads and wide values: more output coordinates (kv_heads * vdim = 640) than one pass of a kernel holds
+    dict(att=dict(heads=8, kv_heads=8, dim=16, vdim=80, scale=0.4, mask={"size": 150}, rot={"dims": 4, "base": 30.0, "scaling": {"factor": 1.0}}),
+         lin=dict(heads=2, dim=24, vdim=8, decay=[0.6, 0.9]),
+         mls=dict(heads=1, dim=16, vdim=16, gate_cap=8.0),
+         moe=dict(ff=16, experts=4, identity=4, groups=2, keep=2, top=2)),
 ]
 _KIND = {"attention": "att", "shared": "att", "lightning": "lin", "mlstm": "mls"}
 

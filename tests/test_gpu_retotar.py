@@ -121,9 +121,11 @@ def build_attention(cfg, i, sub, dtype, dev, cache, source=None):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("portions", [[150], [1, 1, 2, 60, 1, 64, 21], [63, 2, 85], [1] * 40 + [3] + [1] * 70 + [37]])
-@pytest.mark.parametrize("sizes", [0, 1, 2])
-def test_attention_alone_and_on_borrowed_keys(dev, dtype, portions, sizes):
-    """a layer with its own keys and values and a second one that reads the first one's cache with its own queries, mixing matrix and gate"""
+@pytest.mark.parametrize("sizes", [0, 1, 2, 3])
+@pytest.mark.parametrize("kernels", ["matrix cores", "plain, 3 splits"])
+def test_attention_alone_and_on_borrowed_keys(dev, dtype, portions, sizes, kernels):
+    """a layer with its own keys and values and a second one that reads the first one's cache with its own queries, mixing matrix and gate;
+    bf16 portions on the matrix-core kernel (where the sizes allow) or everything on the plain kernel with the window's pages in 3 splits"""
     from zhilight_amd.cache import CacheManager
     cfg = O.small_config(("attention", "shared"), sizes=sizes)
     m0, m1 = cfg["layers"][0]["mixer"], cfg["layers"][1]["mixer"]
@@ -138,6 +140,9 @@ def test_attention_alone_and_on_borrowed_keys(dev, dtype, portions, sizes):
     a0 = build_attention(cfg, 0, s0, dtype, dev, cache)
     a1 = build_attention(cfg, 1, s1, dtype, dev, cache, source=a0)
     assert len(cache.planes) == 2 and a1.k_cache is a0.k_cache
+    for mx in (a0, a1):
+        mx.prompt_kernel = kernels == "matrix cores"
+        mx.n_splits = None if mx.prompt_kernel else 3
     cache.admit("s")
     got0, got1 = feed([a0, a1], cache, h, portions, dev)
     assert rel(got0, ref0) < tol(dtype) and rel(got1, ref1) < tol(dtype)
@@ -158,7 +163,8 @@ def aim_query(sub, m, h, i_star, j_star):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [1, 2, 33, 64, 65, 100])
-def test_window_edges_in_prompts_and_in_decoding(dev, dtype, window):
+@pytest.mark.parametrize("prompt_kernel", [True, False])
+def test_window_edges_in_prompts_and_in_decoding(dev, dtype, window, prompt_kernel):
     """queries aimed at the LAST key the window still holds and at the first one it has dropped, once inside a prompt portion and once
     decoded alone: the first must find its key (nearly all weight), the second must not see it"""
     from zhilight_amd.cache import CacheManager
@@ -186,6 +192,7 @@ def test_window_edges_in_prompts_and_in_decoding(dev, dtype, window):
     cache = CacheManager(320, 2, dev)
     cache.free_pages = [2, 4, 0, 3, 1]
     mix = build_attention(cfg, 0, sub, dtype, dev, cache)
+    mix.prompt_kernel = prompt_kernel
     cache.admit("s")
     (got,) = feed([mix], cache, h, [130, 100] + [1] * 30, dev)
     rows = sorted({**inside, **outside})
@@ -195,7 +202,8 @@ def test_window_edges_in_prompts_and_in_decoding(dev, dtype, window):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("j_star", [0, 1, 63, 64, 65, 127, 128, 200])
-def test_attention_finds_one_far_key_across_pages(dev, dtype, j_star):
+@pytest.mark.parametrize("prompt_kernel", [True, False])
+def test_attention_finds_one_far_key_across_pages(dev, dtype, j_star, prompt_kernel):
     from zhilight_amd.cache import CacheManager
     cfg = O.small_config(("attention",), width=128, sizes=0)
     m = cfg["layers"][0]["mixer"]
@@ -214,6 +222,7 @@ def test_attention_finds_one_far_key_across_pages(dev, dtype, j_star):
     cache = CacheManager(320, 2, dev)
     cache.free_pages = [3, 0, 4, 1, 2]                              # pages out of order
     mix = build_attention(cfg, 0, sub, dtype, dev, cache)
+    mix.prompt_kernel = prompt_kernel
     cache.admit("s")
     (got,) = feed([mix], cache, h, [129, 110] + [1] * 21, dev)      # 230 inside a portion, 259 decoded alone
     assert float(rel_rows(got[[230, 259]], ref[[230, 259]]).max()) < 2 * tol(dtype)

@@ -4,19 +4,21 @@
 //
 // k_rope_norm_store    a workgroup per token, a wave per head in turn: the head's coordinates in registers, rotated, normed, written back
 //                      (queries, fp32, in place) or to the token's row of the paged planes (keys, values; serving format)
-// k_window_attention   a workgroup per (token, query head): keys of the window in chunks of kChunk -- a wave per key for the scores
-//                      (butterfly over the head size), running maximum and sum over chunks, then a thread per output coordinate for P.V.
-//                      With all_kv the weights of a query head are applied to the values of EVERY key / value head: mixing the heads'
+// k_window_attention   a workgroup per (token, query head, split of the window's pages): a page of keys at a time -- a wave per key for the
+//                      scores (butterfly over the head size), running maximum and sum, then a thread per output coordinate for P.V over the
+//                      page's transposed values.  Single decoded tokens in both formats, and everything in fp32.
+// k_window_attention_mfma  bf16 portions on the matrix cores, 64 queries x one head per workgroup (described at the kernel)
+//                      With all_kv both apply the weights of a query head to the values of EVERY key / value head: mixing the heads'
 //                      weights afterwards is then a small product per token (k_head_mix_gate), sum_g T[h][g] acc[g][c(h)], and no weight
 //                      ever has to wait for another head's normaliser.
-// k_head_mix_gate      a workgroup per token: the mix over heads, the turn back by the token's own position, the gate
+// k_head_mix_gate      a workgroup per token: the splits merged, the mix over heads, the turn back by the token's own position, the gate
 // Positions, angles, scores, weights, sums: fp32.  exp / sin / cos are the accurate library versions.
 #include "seq_common.h"
 
 namespace {
 
 constexpr int kMaxE = 8;            // coordinates of a head per lane: dim, vdim <= 64 * kMaxE
-constexpr int kChunk = 128;         // keys per pass of k_window_attention
+constexpr int kChunk = 128;         // the largest page k_window_attention walks
 constexpr int kMaxV = 8;            // output coordinates per thread: (all_kv ? kv_heads : 1) * vdim <= 256 * kMaxV
 
 // one head of `size` coordinates in the lanes' registers (coordinate i in lane i % 64, register i / 64): rotate the first n_rot (pairs
@@ -64,7 +66,8 @@ __global__ __launch_bounds__(256) void k_rope_norm_store(const RopeP p, const zl
     const int posi = b.seq_pos0[sq] + (t - b.seq_start[sq]);
     const float pos = (float)posi;
     float* row = p.proj + (size_t)t * p.ld;
-    const size_t crow = (size_t)b.page_table[(size_t)sq * b.max_pages + posi / b.page_size] * b.page_size + posi % b.page_size;
+    const size_t cpage = (size_t)b.page_table[(size_t)sq * b.max_pages + posi / b.page_size];
+    const size_t crow = cpage * b.page_size + posi % b.page_size;
     const int n_kv = p.k_cache ? p.kv_heads : 0;
     float v[kMaxE];
     for (int h = wave; h < p.heads + 2 * n_kv; h += 4) {                 // (a wave owns its heads: no two waves touch the same numbers)
@@ -85,91 +88,333 @@ __global__ __launch_bounds__(256) void k_rope_norm_store(const RopeP p, const zl
             rope_head(v, row + p.v_col0 + c * p.vdim, p.vdim, p.v_freq ? p.vdim : 0, p.v_freq, pos, false, 0.f, lane);
 #pragma unroll
             for (int r = 0; r < kMaxE; ++r)
-                if (lane + 64 * r < p.vdim) SeqT<DT>::st(p.v_cache, (crow * p.kv_heads + c) * p.vdim + lane + 64 * r, v[r]);
+                if (lane + 64 * r < p.vdim)                             // values lie transposed inside a page: (kv head, coordinate, key)
+                    SeqT<DT>::st(p.v_cache, ((cpage * p.kv_heads + c) * p.vdim + lane + 64 * r) * b.page_size + posi % b.page_size, v[r]);
         }
     }
 }
+
+// 8 consecutive cached numbers as fp32
+template <int DT> struct Ld8;
+template <> struct Ld8<ZL_BF16> {
+    static __device__ __forceinline__ void ld(const void* p, size_t i, float* v) {
+        const uint4 u = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p) + i);
+        const uint32_t q[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = __builtin_bit_cast(float, q[j] << 16);
+            v[2 * j + 1] = __builtin_bit_cast(float, q[j] & 0xffff0000u);
+        }
+    }
+};
+template <> struct Ld8<ZL_F32> {
+    static __device__ __forceinline__ void ld(const void* p, size_t i, float* v) {
+        const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i);
+        const float4 c = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = c.x; v[5] = c.y; v[6] = c.z; v[7] = c.w;
+    }
+};
 
 struct AttnP {
     const float* q; int64_t ldq; int q_col0;
     const void* k_cache; const void* v_cache;
     float scale; int window, heads, kv_heads, dim, vdim, all_kv;
-    float* acc;
+    float* acc; float* ml;                 // (n_tok, heads, n_splits, nv) partial sums | (n_tok, heads, n_splits, 2) their maximum and weight sum
+    int n_splits, pages_per_split, single_only;
+    const int32_t* tiles;                  // the matrix-core kernel: (first flat token, rows, sequence) per query tile
 };
 
+// split s of a token walks the pages first + s * pages_per_split .. of its window (first = the page of the window's oldest key), a page at a
+// time: scores of the page's keys (a wave per key), weights with the running maximum -- 0 for keys outside the window or after the
+// token -- then every thread adds the WHOLE page of its value coordinates (the plane holds values transposed, 8 keys per 16-byte load).
+// What a split leaves is unnormalised: sum_j e^(s_j - m) v_j with m and sum_j e^(s_j - m); k_head_mix_gate merges the splits.
 template <int DT>
 __global__ __launch_bounds__(256) void k_window_attention(const AttnP p, const zls_batch_t b) {
     extern __shared__ float lds[];
     __shared__ float red[16];
-    __shared__ float sc[kChunk];
-    __shared__ int rowi[kChunk];
+    __shared__ __attribute__((aligned(16))) float sc[kChunk];
     float* qs = lds;                                                      // [dim], already times scale
-    const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.x, g = blockIdx.y, sp = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sq = b.tok_seq[t];
+    if (p.single_only && b.seq_start[sq + 1] - b.seq_start[sq] > 1) return;
+    const int ps = b.page_size;
     const int pos = b.seq_pos0[sq] + (t - b.seq_start[sq]);
     const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
     const int c = g / (p.heads / p.kv_heads);
     const int nv = p.all_kv ? p.kv_heads * p.vdim : p.vdim, voff = p.all_kv ? 0 : c * p.vdim;
     const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
+    const int pg0 = lo / ps + sp * p.pages_per_split, pg1 = min(pos / ps, pg0 + p.pages_per_split - 1);
     for (int i = tid; i < p.dim; i += 256) qs[i] = p.q[(size_t)t * p.ldq + p.q_col0 + g * p.dim + i] * p.scale;
     float A[kMaxV];
 #pragma unroll
     for (int r = 0; r < kMaxV; ++r) A[r] = 0.f;
     float m = -INFINITY, l = 0.f;
     __syncthreads();
-    for (int j0 = lo; j0 <= pos; j0 += kChunk) {
-        const int cn = min(kChunk, pos - j0 + 1);
-        for (int jj = wave; jj < cn; jj += 4) {
+    for (int pg = pg0; pg <= pg1; ++pg) {
+        const size_t page = (size_t)pages[pg];
+        const int j0 = pg * ps;
+        for (int jj = wave; jj < ps; jj += 4) {
             const int j = j0 + jj;
-            const size_t row = (size_t)pages[j / b.page_size] * b.page_size + j % b.page_size;
-            const size_t at = (row * p.kv_heads + c) * p.dim;
-            float part = 0.f;
-            for (int i = lane; i < p.dim; i += 64) part = fmaf(qs[i], SeqT<DT>::ld(p.k_cache, at + i), part);
-            part = zl_wave_sum(part);
-            if (lane == 0) { sc[jj] = part; rowi[jj] = (int)row; }
+            float part = -INFINITY;
+            if (j >= lo && j <= pos) {                                    // (wave-uniform)
+                const size_t at = ((page * ps + jj) * p.kv_heads + c) * p.dim;
+                part = 0.f;
+                for (int i = lane; i < p.dim; i += 64) part = fmaf(qs[i], SeqT<DT>::ld(p.k_cache, at + i), part);
+                part = zl_wave_sum(part);
+            }
+            if (lane == 0) sc[jj] = part;
         }
         __syncthreads();
         float cm = -INFINITY;
-        for (int jj = tid; jj < cn; jj += 256) cm = fmaxf(cm, sc[jj]);
-        const float m_new = fmaxf(m, zl_block_max(cm, red));
-        float ps = 0.f;
-        for (int jj = tid; jj < cn; jj += 256) { const float e = expf(sc[jj] - m_new); sc[jj] = e; ps += e; }
-        const float corr = expf(m - m_new);                               // (first chunk: exp(-inf) = 0 on zero sums)
-        l = l * corr + zl_block_sum(ps, red);                             // (its barriers also publish the weights in sc[])
+        for (int jj = tid; jj < ps; jj += 256) cm = fmaxf(cm, sc[jj]);
+        const float m_new = fmaxf(m, zl_block_max(cm, red));              // finite: the page holds a key of the window
+        float psum = 0.f;
+        for (int jj = tid; jj < ps; jj += 256) { const float e = expf(sc[jj] - m_new); sc[jj] = e; psum += e; }      // e^(-inf) = 0
+        const float corr = expf(m - m_new);                               // (first page: 0, on sums that are 0)
+        l = l * corr + zl_block_sum(psum, red);                           // (its barriers also publish the weights in sc[])
         m = m_new;
 #pragma unroll
         for (int r = 0; r < kMaxV; ++r) {
             const int e = tid + 256 * r;
             if (e < nv) {
                 float a = A[r] * corr;
-                for (int jj = 0; jj < cn; ++jj)
-                    a = fmaf(sc[jj], SeqT<DT>::ld(p.v_cache, (size_t)rowi[jj] * p.kv_heads * p.vdim + voff + e), a);
+                const size_t at = (page * p.kv_heads * p.vdim + voff + e) * ps;
+                for (int j8 = 0; j8 < ps; j8 += 8) {
+                    float v[8];
+                    Ld8<DT>::ld(p.v_cache, at + j8, v);
+                    const float4 w0 = *reinterpret_cast<const float4*>(sc + j8), w1 = *reinterpret_cast<const float4*>(sc + j8 + 4);
+                    a = fmaf(w0.x, v[0], a); a = fmaf(w0.y, v[1], a); a = fmaf(w0.z, v[2], a); a = fmaf(w0.w, v[3], a);
+                    a = fmaf(w1.x, v[4], a); a = fmaf(w1.y, v[5], a); a = fmaf(w1.z, v[6], a); a = fmaf(w1.w, v[7], a);
+                }
                 A[r] = a;
             }
         }
-        __syncthreads();                                                  // sc[] / rowi[] are free for the next chunk
+        __syncthreads();                                                  // sc[] is free for the next page
     }
-    const float inv = 1.0f / l;
-    float* out = p.acc + ((size_t)t * p.heads + g) * nv;
+    const size_t at = ((size_t)t * p.heads + g) * p.n_splits + sp;
+    float* out = p.acc + at * nv;
 #pragma unroll
     for (int r = 0; r < kMaxV; ++r)
-        if (tid + 256 * r < nv) out[tid + 256 * r] = A[r] * inv;
+        if (tid + 256 * r < nv) out[tid + 256 * r] = A[r];
+    if (tid == 0) { p.ml[2 * at] = m; p.ml[2 * at + 1] = l; }            // (a split without pages: -inf, 0, sums 0)
+}
+
+// ---- portions on the matrix cores (bf16, 64-key pages) ------------------------------------------------------------------------------------
+// A workgroup = a tile of up to 64 consecutive queries of one sequence x one query head (x a part of the output coordinates when they
+// are many); wave w owns queries 16 w .. for the scores and the softmax, and a share of the (kv head, 16 value coordinates) output blocks
+// for ALL 64 queries.  Per page of keys:
+//   S^T = K Q^T      v_mfma_f32_16x16x32_bf16, A = 16 keys x 32 coordinates straight from the cache rows (16 bytes a lane), B = the wave's
+//                    queries, split once into bf16 halves hi + lo (two MFMAs: the scores keep the fp32 queries' bits)
+//   softmax          a lane holds 16 scores of one query (keys 4 kq + r of the page's four 16-key blocks); maximum and sum over the four
+//                    lanes of the query by two butterflies; running maximum, correction e^(m_old - m_new)
+//   P -> LDS         the weights, split into bf16 halves, in exactly the registers' order: a lane's 8 numbers for 32 keys ARE the B operand
+//                    of O^T = V^T P^T if slot i of quarter kq means key 4 kq + i (i < 4) or 16 + 4 kq + i - 4 -- so the A operand takes V^T
+//                    in that order: two 8-byte loads from the transposed value plane
+//   O^T += V^T P^T   every wave: its output blocks x 4 query blocks x 2 key halves x (hi, lo), after scaling by the queries' corrections
+// Two P buffers alternate, so one barrier per page is enough.
+typedef __bf16 b8v __attribute__((ext_vector_type(8)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+constexpr int kItems = 8;               // output blocks (16 value coordinates of one kv head) per wave: 4 waves x 8 x 16 = 512 per workgroup
+
+__device__ __forceinline__ uint32_t bf16_bits(float f) {                 // round to nearest even; finite inputs
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ void split8(const float* v, uint4& hi, uint4& lo) {
+    uint32_t h[8], l[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        h[i] = bf16_bits(v[i]);
+        l[i] = bf16_bits(v[i] - __builtin_bit_cast(float, h[i] << 16));
+    }
+    hi = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+    lo = make_uint4(l[0] | l[1] << 16, l[2] | l[3] << 16, l[4] | l[5] << 16, l[6] | l[7] << 16);
+}
+
+template <int KS>                       // 32-coordinate steps of the head size: dim <= 32 KS
+__global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, const zls_batch_t b) {
+    __shared__ uint4 pfrag[2][4][2][2][64];                              // [buffer][query block][key half][hi, lo][lane]
+    __shared__ float corr_s[2][64], l_s[64];
+    const int tile = blockIdx.x, g = blockIdx.y, part = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nrow = lane & 15, kq = lane >> 4;
+    const int t0 = p.tiles[3 * tile], rows = p.tiles[3 * tile + 1], sq = p.tiles[3 * tile + 2];
+    const int pos0 = b.seq_pos0[sq] + (t0 - b.seq_start[sq]);
+    const int G = p.kv_heads, d = p.dim, vd = p.vdim;
+    const int c = g / (p.heads / G);
+    const int nv = p.all_kv ? G * vd : vd;
+    const int32_t* pages = b.page_table + (size_t)sq * b.max_pages;
+    const uint16_t* kc = reinterpret_cast<const uint16_t*>(p.k_cache);
+    const uint16_t* vc = reinterpret_cast<const uint16_t*>(p.v_cache);
+    // the wave's own query (for the scores): tile row 16 wave + nrow
+    const int qi = 16 * wave + nrow;
+    const bool qok = qi < rows;
+    const int pq = pos0 + qi;
+    uint4 qh[KS], ql[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int x = 32 * ks + 8 * kq + i;
+            v[i] = (qok && x < d) ? p.q[(size_t)(t0 + qi) * p.ldq + p.q_col0 + g * d + x] * p.scale : 0.f;
+        }
+        split8(v, qh[ks], ql[ks]);
+    }
+    // this wave's output blocks: block index nb = (part * 4 * kItems) + wave + 4 i  ->  (kv head, 16 coordinates)
+    const int n_blocks = nv / 16, vb_per = vd / 16;
+    f4v acc[kItems][4];
+#pragma unroll
+    for (int i = 0; i < kItems; ++i)
+#pragma unroll
+        for (int qb = 0; qb < 4; ++qb) acc[i][qb] = (f4v){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    const int lo_key = p.window > 0 ? max(0, pos0 - p.window + 1) : 0, hi_key = pos0 + rows - 1;
+    int buf = 0;
+    for (int pg = lo_key / 64; pg <= hi_key / 64; ++pg, buf ^= 1) {
+        const size_t page = (size_t)pages[pg];
+        // ---- scores of the wave's 16 queries against the page's 64 keys
+        f4v st[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            st[kb] = (f4v){0.f, 0.f, 0.f, 0.f};
+            const uint16_t* kr = kc + ((page * 64 + kb * 16 + nrow) * G + c) * d + 8 * kq;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const uint4 kf = (32 * ks + 8 * kq < d) ? *reinterpret_cast<const uint4*>(kr + 32 * ks) : make_uint4(0, 0, 0, 0);
+                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, kf), __builtin_bit_cast(b8v, qh[ks]), st[kb], 0, 0, 0);
+                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, kf), __builtin_bit_cast(b8v, ql[ks]), st[kb], 0, 0, 0);
+            }
+        }
+        // st[kb][r]: key pg * 64 + 16 kb + 4 kq + r, query nrow
+        float cm = -INFINITY;
+        bool vis[4][4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = pg * 64 + 16 * kb + 4 * kq + r;
+                vis[kb][r] = qok && j <= pq && (p.window <= 0 || pq - j < p.window);
+                if (vis[kb][r]) cm = fmaxf(cm, st[kb][r]);
+            }
+        cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+        cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        const float m_new = fmaxf(m_run, cm);
+        const float corr = m_new == -INFINITY ? 1.0f : expf(m_run - m_new);
+        float pw[4][4], psum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                pw[kb][r] = vis[kb][r] ? expf(st[kb][r] - m_new) : 0.f;
+                psum += pw[kb][r];
+            }
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+            const float v[8] = {pw[2 * h2][0], pw[2 * h2][1], pw[2 * h2][2], pw[2 * h2][3],
+                                pw[2 * h2 + 1][0], pw[2 * h2 + 1][1], pw[2 * h2 + 1][2], pw[2 * h2 + 1][3]};
+            uint4 hi, lo;
+            split8(v, hi, lo);
+            pfrag[buf][wave][h2][0][lane] = hi;
+            pfrag[buf][wave][h2][1][lane] = lo;
+        }
+        if (kq == 0) corr_s[buf][qi] = corr;
+        __syncthreads();
+        // ---- O^T += V^T P^T for this wave's output blocks and all four query blocks
+        float cq[4];
+#pragma unroll
+        for (int qb = 0; qb < 4; ++qb) cq[qb] = corr_s[buf][16 * qb + nrow];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i)
+#pragma unroll
+            for (int qb = 0; qb < 4; ++qb) acc[i][qb] *= cq[qb];
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+            uint4 vf[kItems];
+#pragma unroll
+            for (int i = 0; i < kItems; ++i) {
+                const int nb = part * 4 * kItems + wave + 4 * i;
+                vf[i] = make_uint4(0, 0, 0, 0);
+                if (nb < n_blocks) {
+                    const int cc = p.all_kv ? nb / vb_per : c, x = (nb % vb_per) * 16 + nrow;
+                    const uint16_t* vr = vc + ((page * G + cc) * vd + x) * 64 + 32 * h2 + 4 * kq;
+                    const uint2 a0 = *reinterpret_cast<const uint2*>(vr), a1 = *reinterpret_cast<const uint2*>(vr + 16);
+                    vf[i] = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                }
+            }
+#pragma unroll
+            for (int qb = 0; qb < 4; ++qb) {
+                const uint4 bh = pfrag[buf][qb][h2][0][lane], bl = pfrag[buf][qb][h2][1][lane];
+#pragma unroll
+                for (int i = 0; i < kItems; ++i) {
+                    acc[i][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, vf[i]), __builtin_bit_cast(b8v, bh), acc[i][qb], 0, 0, 0);
+                    acc[i][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, vf[i]), __builtin_bit_cast(b8v, bl), acc[i][qb], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (kq == 0) l_s[qi] = l_run;
+    __syncthreads();
+    // acc[i][qb][r]: value coordinate 16 (block) + 4 kq + r of query 16 qb + nrow; split 0 of the token's partial sums, already normalised
+#pragma unroll
+    for (int qb = 0; qb < 4; ++qb) {
+        const int row = 16 * qb + nrow;
+        if (row >= rows) continue;
+        const float inv = 1.0f / l_s[row];
+        float* out = p.acc + (((size_t)(t0 + row) * p.heads + g) * p.n_splits) * nv;
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            const int nb = part * 4 * kItems + wave + 4 * i;
+            if (nb < n_blocks)
+                *reinterpret_cast<float4*>(out + nb * 16 + 4 * kq) = make_float4(acc[i][qb][0] * inv, acc[i][qb][1] * inv, acc[i][qb][2] * inv, acc[i][qb][3] * inv);
+        }
+    }
+    if (part == 0)
+        for (int e = tid; e < rows * p.n_splits; e += 256) {
+            const int row = e / p.n_splits, sp = e % p.n_splits;
+            float* mlp = p.ml + 2 * ((((size_t)(t0 + row) * p.heads + g) * p.n_splits) + sp);
+            mlp[0] = sp == 0 ? 0.f : -INFINITY;
+            mlp[1] = sp == 0 ? 1.f : 0.f;
+        }
 }
 
 struct MixP {
-    const float* acc; const float* talk; const float* v_freq; const float* gate; int64_t ldg; int g_col0;
-    int heads, kv_heads, vdim;
+    const float* acc; const float* ml; const float* talk; const float* v_freq; const float* gate; int64_t ldg; int g_col0;
+    int heads, kv_heads, vdim, n_splits;
     void* out;
 };
 
+// a workgroup per token: the splits of every head merged (weights e^(m_s - M) / L into LDS), the mix over heads, the turn back by the
+// token's own position, the gate
 template <int DT>
 __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_batch_t b) {
+    extern __shared__ float wsp[];                                        // [heads][n_splits]
     const int t = blockIdx.x;
     const int sq = b.tok_seq[t];
     const float pos = (float)(b.seq_pos0[sq] + (t - b.seq_start[sq]));
-    const int per = p.heads / p.kv_heads, half = p.vdim >> 1;
-    const int nv = p.talk ? p.kv_heads * p.vdim : p.vdim;                 // a head's stride in acc
-    const float* a = p.acc + (size_t)t * p.heads * nv;
+    const int per = p.heads / p.kv_heads, half = p.vdim >> 1, S = p.n_splits;
+    const int nv = p.talk ? p.kv_heads * p.vdim : p.vdim;                 // a head's stride in a split of acc
+    const float* a = p.acc + (size_t)t * p.heads * S * nv;
+    for (int g = threadIdx.x; g < p.heads; g += 256) {
+        const float* mlp = p.ml + 2 * ((size_t)t * p.heads + g) * S;
+        float M = -INFINITY, L = 0.f;
+        for (int s = 0; s < S; ++s) M = fmaxf(M, mlp[2 * s]);
+        for (int s = 0; s < S; ++s) L += mlp[2 * s + 1] * expf(mlp[2 * s] - M);
+        for (int s = 0; s < S; ++s) wsp[g * S + s] = mlp[2 * s + 1] > 0.f ? expf(mlp[2 * s] - M) / L : 0.f;
+    }
+    __syncthreads();
+    auto merged = [&](int g, int col) {                                   // head g's sum for column col of its nv
+        float v = 0.f;
+        for (int s = 0; s < S; ++s) {
+            const float w = wsp[g * S + s];
+            if (w != 0.f) v = fmaf(w, a[((size_t)g * S + s) * nv + col], v);
+        }
+        return v;
+    };
     // a thread owns a PAIR (m, m + vdim / 2) of one head (an odd vdim without rotation: the last coordinate alone)
     const int pairs = p.v_freq ? half : (p.vdim + 1) / 2;
     for (int w = threadIdx.x; w < p.heads * pairs; w += 256) {
@@ -180,13 +425,12 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
             const int c = h / per;
             for (int g = 0; g < p.heads; ++g) {
                 const float tw = p.talk[h * p.heads + g];
-                const float* ag = a + (size_t)g * nv + c * p.vdim;
-                u = fmaf(tw, ag[i0], u);
-                if (i1 < p.vdim) v = fmaf(tw, ag[i1], v);
+                u = fmaf(tw, merged(g, c * p.vdim + i0), u);
+                if (i1 < p.vdim) v = fmaf(tw, merged(g, c * p.vdim + i1), v);
             }
         } else {
-            u = a[(size_t)h * nv + i0];
-            if (i1 < p.vdim) v = a[(size_t)h * nv + i1];
+            u = merged(h, i0);
+            if (i1 < p.vdim) v = merged(h, i1);
         }
         if (p.v_freq) {
             float sn, cs;
@@ -228,29 +472,61 @@ extern "C" int zls_rope_norm_store(float* proj, int64_t ld, int64_t q_col0, int6
 
 extern "C" int zls_window_attention(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache, const zls_batch_t* b,
                                     float scale, int64_t window, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc,
-                                    int dtype, zl_stream_t s) {
-    ZL_CHECK_ARG(q && k_cache && v_cache && acc && seq_batch_ok(b) && b->page_table && b->page_size > 0, ZL_EINVAL);
+                                    float* ml, int64_t n_splits, int64_t pages_per_split, int single_only, int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(q && k_cache && v_cache && acc && ml && seq_batch_ok(b) && b->page_table && b->page_size > 0, ZL_EINVAL);
     ZL_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && heads <= 65535, ZL_ESHAPE);
-    ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && window < (1 << 30), ZL_ESHAPE);
-    ZL_CHECK_ARG((all_kv ? kv_heads : 1) * vdim <= 256 * kMaxV && dim <= 8192, ZL_ELIMIT);
-    AttnP p;
+    ZL_CHECK_ARG(q_col0 >= 0 && q_col0 + heads * dim <= ldq && window < (1 << 30) && n_splits >= 1 && n_splits <= 65535 && pages_per_split >= 1,
+                 ZL_ESHAPE);
+    ZL_CHECK_ARG((all_kv ? kv_heads : 1) * vdim <= 256 * kMaxV && dim <= 8192 && b->page_size <= kChunk && b->page_size % 8 == 0, ZL_ELIMIT);
+    AttnP p = {};
     p.q = q; p.ldq = ldq; p.q_col0 = (int)q_col0; p.k_cache = k_cache; p.v_cache = v_cache; p.scale = scale; p.window = (int)window;
-    p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.all_kv = all_kv ? 1 : 0; p.acc = acc;
+    p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.all_kv = all_kv ? 1 : 0; p.acc = acc; p.ml = ml;
+    p.n_splits = (int)n_splits; p.pages_per_split = (int)pages_per_split; p.single_only = single_only ? 1 : 0;
     const size_t lds = (size_t)dim * sizeof(float);
-#define CALL(DT) hipLaunchKernelGGL((k_window_attention<DT>), dim3(b->n_tok, (unsigned)heads), dim3(256), lds, (hipStream_t)s, p, *b);
+#define CALL(DT) hipLaunchKernelGGL((k_window_attention<DT>), dim3(b->n_tok, (unsigned)heads, (unsigned)n_splits), dim3(256), lds, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();
 }
 
-extern "C" int zls_head_mix_gate(const float* acc, const float* talk, const float* v_freq, const float* gate, int64_t ldg, int64_t g_col0,
-                                 const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out, int dtype, zl_stream_t s) {
-    ZL_CHECK_ARG(acc && out && seq_batch_ok(b) && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0, ZL_EINVAL);
+extern "C" int zls_window_attention_prompt(const float* q, int64_t ldq, int64_t q_col0, const void* k_cache, const void* v_cache,
+                                           const zls_batch_t* b, const int32_t* tiles, int64_t n_tiles, float scale, int64_t window, int64_t heads,
+                                           int64_t kv_heads, int64_t dim, int64_t vdim, int all_kv, float* acc, float* ml, int64_t n_splits,
+                                           int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(q && k_cache && v_cache && acc && ml && tiles && n_tiles > 0 && seq_batch_ok(b) && b->page_table, ZL_EINVAL);
+    ZL_CHECK_ARG(dtype == ZL_BF16, ZL_EDTYPE);
+    ZL_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads <= 65535 && n_splits >= 1 && q_col0 >= 0 && q_col0 + heads * dim <= ldq,
+                 ZL_ESHAPE);
+    ZL_CHECK_ARG(b->page_size == 64 && dim > 0 && dim % 8 == 0 && dim <= 256 && vdim > 0 && vdim % 16 == 0 && window < (1 << 30), ZL_ESHAPE);
+    AttnP p = {};
+    p.q = q; p.ldq = ldq; p.q_col0 = (int)q_col0; p.k_cache = k_cache; p.v_cache = v_cache; p.scale = scale; p.window = (int)window;
+    p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.dim = (int)dim; p.vdim = (int)vdim; p.all_kv = all_kv ? 1 : 0; p.acc = acc; p.ml = ml;
+    p.n_splits = (int)n_splits; p.tiles = tiles;
+    const int64_t n_blocks = (all_kv ? kv_heads : 1) * vdim / 16, parts = (n_blocks + 4 * kItems - 1) / (4 * kItems);
+    ZL_CHECK_ARG(parts <= 65535, ZL_ELIMIT);
+    const dim3 grid((unsigned)n_tiles, (unsigned)heads, (unsigned)parts);
+    hipStream_t hs = (hipStream_t)s;
+    const int ks = (int)((dim + 31) / 32);
+    if (ks <= 1) hipLaunchKernelGGL((k_window_attention_mfma<1>), grid, dim3(256), 0, hs, p, *b);
+    else if (ks <= 2) hipLaunchKernelGGL((k_window_attention_mfma<2>), grid, dim3(256), 0, hs, p, *b);
+    else if (ks <= 3) hipLaunchKernelGGL((k_window_attention_mfma<3>), grid, dim3(256), 0, hs, p, *b);
+    else if (ks <= 4) hipLaunchKernelGGL((k_window_attention_mfma<4>), grid, dim3(256), 0, hs, p, *b);
+    else if (ks <= 6) hipLaunchKernelGGL((k_window_attention_mfma<6>), grid, dim3(256), 0, hs, p, *b);
+    else hipLaunchKernelGGL((k_window_attention_mfma<8>), grid, dim3(256), 0, hs, p, *b);
+    return zl_launch_status();
+}
+
+extern "C" int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_splits, const float* talk, const float* v_freq, const float* gate,
+                                 int64_t ldg, int64_t g_col0, const zls_batch_t* b, int64_t heads, int64_t kv_heads, int64_t vdim, void* out,
+                                 int dtype, zl_stream_t s) {
+    ZL_CHECK_ARG(acc && ml && out && seq_batch_ok(b) && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0 && n_splits >= 1, ZL_EINVAL);
     ZL_CHECK_ARG((!v_freq || vdim % 2 == 0) && (!gate || (g_col0 >= 0 && g_col0 + heads * vdim <= ldg)), ZL_ESHAPE);
+    const size_t lds = (size_t)heads * n_splits * sizeof(float);
+    ZL_CHECK_ARG(lds <= 60 * 1024, ZL_ELIMIT);
     MixP p;
-    p.acc = acc; p.talk = talk; p.v_freq = v_freq; p.gate = gate; p.ldg = ldg; p.g_col0 = (int)g_col0; p.heads = (int)heads;
-    p.kv_heads = (int)kv_heads; p.vdim = (int)vdim; p.out = out;
-#define CALL(DT) hipLaunchKernelGGL((k_head_mix_gate<DT>), dim3(b->n_tok), dim3(256), 0, (hipStream_t)s, p, *b);
+    p.acc = acc; p.ml = ml; p.n_splits = (int)n_splits; p.talk = talk; p.v_freq = v_freq; p.gate = gate; p.ldg = ldg; p.g_col0 = (int)g_col0;
+    p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.vdim = (int)vdim; p.out = out;
+#define CALL(DT) hipLaunchKernelGGL((k_head_mix_gate<DT>), dim3(b->n_tok), dim3(256), lds, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();

@@ -207,6 +207,8 @@ class WindowAttention:
         self.eps, self.qk_norm, self.rotate_values, self.has_talk, self.has_gate = float(eps), qk_norm, rotate_values, talk, gate
         self.kv_source = kv_source
         self.k_cache = self.v_cache = None
+        self.prompt_kernel = True         # bf16 portions on the matrix-core kernel (False: everything on the plain kernel)
+        self.n_splits = None              # workgroups per (token, head) of the plain kernel (None: enough to fill the chip)
 
     def _cols(self):
         H, G, d, v = self.heads, self.kv_heads, self.dim, self.vdim
@@ -245,7 +247,7 @@ class WindowAttention:
             self.k_cache, self.v_cache = self.kv_source.k_cache, self.kv_source.v_cache
             return
         self.k_cache = cache.add_plane(self.name + ".k", (self.kv_heads * self.dim,), dtype)
-        self.v_cache = cache.add_plane(self.name + ".v", (self.kv_heads * self.vdim,), dtype)
+        self.v_cache = cache.add_plane(self.name + ".v", (self.kv_heads * self.vdim,), dtype)      # (the kernels keep a page transposed)
 
     def weight_bytes(self):
         return sum(t.numel() * t.element_size() for t in (self.w_in, self.w_o))
@@ -257,8 +259,9 @@ class WindowAttention:
         proj = seqops.gemm_nt(h, self.w_in)                                       # fp32 [q | k | v | gate]
         seqops.rope_norm_store(proj, 0, k0, v0, H, G, d, v, self.qk_freq, self.rot_dims, self.v_freq, self.eps, self.qk_norm, batch,
                                self.k_cache if own else None, self.v_cache if own else None)
-        acc = seqops.window_attention(proj, 0, self.k_cache, self.v_cache, batch, self.scale, self.window, H, G, d, v, all_kv=self.has_talk)
-        a = seqops.head_mix_gate(acc, self.talk, self.v_freq, proj if self.has_gate else None, g0, batch, H, G, v, h.dtype)
+        acc, ml, n_splits = seqops.window_attention(proj, 0, self.k_cache, self.v_cache, batch, self.scale, self.window, H, G, d, v,
+                                                    all_kv=self.has_talk, mfma=self.prompt_kernel, n_splits=self.n_splits)
+        a = seqops.head_mix_gate(acc, ml, n_splits, self.talk, self.v_freq, proj if self.has_gate else None, g0, batch, H, G, v, h.dtype)
         return seqops.gemm_nt(a, self.w_o)
 
 

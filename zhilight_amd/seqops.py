@@ -18,7 +18,7 @@ SO_PATH = os.path.join(_HERE, "libzhilight_amd_seq.so")
 SYMBOLS = ["zls_version", "zls_gemm_nt", "zls_embed", "zls_token_shift", "zls_add_scalar_norm", "zls_scalar_norm_rows", "zls_polynorm",
            "zls_latent_store", "zls_latent_attention", "zls_latent_attention_workspace_bytes", "zls_latent_attention_prompt", "zls_gemm_nt_gather",
            "zls_conv_silu", "zls_conv_tail_update", "zls_ssm_scan", "zls_ssm_scan_workspace_bytes", "zls_gated_group_norm", "zls_layer_norm",
-           "zls_add_layer_norm", "zls_rope_norm_store", "zls_window_attention", "zls_head_mix_gate", "zls_decay_scan", "zls_exp_gates",
+           "zls_add_layer_norm", "zls_rope_norm_store", "zls_window_attention", "zls_window_attention_prompt", "zls_head_mix_gate", "zls_decay_scan", "zls_exp_gates",
            "zls_linear_attn_finish", "zls_moe_route", "zls_moe_align", "zls_gemm_nt_grouped", "zls_silu_mul", "zls_moe_combine"]
 _STATUS = {-1: "invalid argument (null pointer / non-positive size)", -2: "shape not supported", -3: "dtype not supported",
            -4: "exceeds a hardware limit"}
@@ -118,8 +118,15 @@ class RaggedBatch:
             n = pos0 + count
             rows = [pages[j // page_size] * page_size + j % page_size for j in range(n)]
             ctx_rows += rows + [rows[0]] * (-n % 64)
-        # ONE host array, one copy: [seq_start | seq_pos0 | seq_slot | tok_seq | page_table | ctx_start | ctx_rows]
-        host = torch.tensor(starts + [s[1] for s in seqs] + [s[2] for s in seqs] + tok_seq + table + ctx_start + ctx_rows, dtype=torch.int32)
+        # query tiles of the portions: (first flat token, rows <= 64, sequence) -- what the matrix-core attention kernels walk
+        q_tiles = []
+        for i, (count, pos0, slot, pages) in enumerate(seqs):
+            if count > 1:
+                for r0 in range(0, count, 64):
+                    q_tiles += [starts[i] + r0, min(64, count - r0), i]
+        # ONE host array, one copy: [seq_start | seq_pos0 | seq_slot | tok_seq | page_table | ctx_start | ctx_rows | q_tiles]
+        host = torch.tensor(starts + [s[1] for s in seqs] + [s[2] for s in seqs] + tok_seq + table + ctx_start + ctx_rows + q_tiles,
+                            dtype=torch.int32)
         self.dev = host.to(device, non_blocking=False)
         o = [0, n_seq + 1, 2 * n_seq + 1, 3 * n_seq + 1, 3 * n_seq + 1 + starts[-1]]
         base = self.dev.data_ptr()
@@ -129,6 +136,9 @@ class RaggedBatch:
         self.ctx_start = self.dev[at:at + n_seq]
         self.ctx_rows = self.dev[at + n_seq:at + n_seq + len(ctx_rows)]
         self.n_ctx = len(ctx_rows)
+        self.q_tiles = self.dev[at + n_seq + len(ctx_rows):]
+        self.n_q_tiles = len(q_tiles) // 3
+        self.min_pos0 = min(s[1] for s in seqs)
         self.n_single = sum(1 for c in self.counts if c == 1)
         self.max_ctx = max(s[0] + s[1] for s in seqs)
         self.c = Batch(n_seq, self.n_tok, max_pages, page_size, max(self.counts), 0, *[base + 4 * x for x in o])
@@ -345,36 +355,58 @@ def rope_norm_store(proj, q_col0, k_col0, v_col0, heads, kv_heads, dim, vdim, qk
     if k_cache is not None:
         if tuple(k_cache.shape[1:]) != (batch.c.page_size, kv_heads * dim) or tuple(v_cache.shape[1:]) != (batch.c.page_size, kv_heads * vdim) \
                 or k_cache.dtype != v_cache.dtype:
-            raise ZLError("rope_norm_store: planes must be (pages, page_size, kv_heads * dim | vdim)")
+            raise ZLError("rope_norm_store: planes must be (pages, page_size, kv_heads * dim | vdim)")   # (the value plane's pages are
+            # written transposed, (kv_heads * vdim, page_size): the same bytes of the same plane)
     code = dt_code(k_cache.dtype) if k_cache is not None else F32
     check(lib().zls_rope_norm_store(_p(proj), _i(proj.shape[1]), _i(q_col0), _i(k_col0), _i(v_col0), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
                                     _p(qk_freq), _i(rot_dims), _p(v_freq), _f(eps), C.c_int(int(qk_norm)), batch.ref, _p(k_cache), _p(v_cache),
                                     C.c_int(code), _stream()), "rope_norm_store")
 
 
-def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, kv_heads, dim, vdim, all_kv):
-    """fp32 (n_tok, heads, [kv_heads,] vdim): every query head's softmax weights applied to its own (all_kv False) or every kv head's values"""
+def window_attention(q, q_col0, k_cache, v_cache, batch, scale, window, heads, kv_heads, dim, vdim, all_kv, mfma=True, n_splits=None):
+    """Every query head's softmax weights applied to its own (all_kv False) or every kv head's values.  Returns (acc, ml, n_splits) for
+    head_mix_gate: fp32 partial sums (n_tok, heads, n_splits, nv) and their (maximum, weight sum).  bf16 portions run on the matrix cores
+    when the sizes allow (mfma=False: everything on the plain kernel); single tokens are split over their window's pages."""
     _cuda(q, k_cache, v_cache)
     _f32(q)
-    if tuple(k_cache.shape[1:]) != (batch.c.page_size, kv_heads * dim) or tuple(v_cache.shape[1:]) != (batch.c.page_size, kv_heads * vdim):
+    ps = batch.c.page_size
+    if tuple(k_cache.shape[1:]) != (ps, kv_heads * dim) or tuple(v_cache.shape[1:]) != (ps, kv_heads * vdim) or k_cache.dtype != v_cache.dtype:
         raise ZLError("window_attention: planes must be (pages, page_size, kv_heads * dim | vdim)")
-    acc = torch.empty((batch.n_tok, heads, kv_heads if all_kv else 1, vdim), dtype=torch.float32, device=q.device)
-    check(lib().zls_window_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _f(scale), _i(window), _i(heads),
-                                     _i(kv_heads), _i(dim), _i(vdim), C.c_int(int(all_kv)), _p(acc), C.c_int(dt_code(k_cache.dtype)), _stream()),
-          "window_attention")
-    return acc
+    nv = (kv_heads if all_kv else 1) * vdim
+    prompt = mfma and batch.n_q_tiles > 0 and k_cache.dtype == torch.bfloat16 and ps == 64 and dim % 8 == 0 and dim <= 256 and vdim % 16 == 0
+    plain_tokens = batch.n_single if prompt else batch.n_tok
+    # the pages a window can touch, and enough workgroups to fill the chip (256 CUs, a few per CU) when few tokens take the plain kernel
+    span = min(batch.max_ctx, window) if window > 0 else batch.max_ctx
+    pages = min((span + ps - 2) // ps + 1, (batch.max_ctx + ps - 1) // ps)
+    if n_splits is None:
+        n_splits = 1 if plain_tokens == 0 else max(1, min(pages, 1024 // (plain_tokens * heads)))
+    n_splits = max(1, min(int(n_splits), pages))
+    per = (pages + n_splits - 1) // n_splits
+    acc = torch.empty((batch.n_tok, heads, n_splits, nv), dtype=torch.float32, device=q.device)
+    ml = torch.empty((batch.n_tok, heads, n_splits, 2), dtype=torch.float32, device=q.device)
+    code = C.c_int(dt_code(k_cache.dtype))
+    if prompt:
+        check(lib().zls_window_attention_prompt(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _p(batch.q_tiles),
+                                                _i(batch.n_q_tiles), _f(scale), _i(window), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
+                                                C.c_int(int(all_kv)), _p(acc), _p(ml), _i(n_splits), code, _stream()), "window_attention_prompt")
+    if plain_tokens:
+        check(lib().zls_window_attention(_p(q), _i(q.shape[1]), _i(q_col0), _p(k_cache), _p(v_cache), batch.ref, _f(scale), _i(window), _i(heads),
+                                         _i(kv_heads), _i(dim), _i(vdim), C.c_int(int(all_kv)), _p(acc), _p(ml), _i(n_splits), _i(per),
+                                         C.c_int(int(prompt)), code, _stream()), "window_attention")
+    return acc, ml, n_splits
 
 
-def head_mix_gate(acc, talk, v_freq, gate, g_col0, batch, heads, kv_heads, vdim, dtype):
-    _cuda(acc, talk, v_freq, gate)
-    _f32(acc, talk, v_freq, gate)
+def head_mix_gate(acc, ml, n_splits, talk, v_freq, gate, g_col0, batch, heads, kv_heads, vdim, dtype):
+    _cuda(acc, ml, talk, v_freq, gate)
+    _f32(acc, ml, talk, v_freq, gate)
     if talk is not None and tuple(talk.shape) != (heads, heads):
         raise ZLError("head_mix_gate: the mixing matrix is (heads, heads)")
-    if acc.numel() != batch.n_tok * heads * (kv_heads if talk is not None else 1) * vdim:
-        raise ZLError("head_mix_gate: acc does not fit")
+    if acc.numel() != batch.n_tok * heads * n_splits * (kv_heads if talk is not None else 1) * vdim or ml.numel() != batch.n_tok * heads * n_splits * 2:
+        raise ZLError("head_mix_gate: acc / ml do not fit")
     out = torch.empty((batch.n_tok, heads * vdim), dtype=dtype, device=acc.device)
-    check(lib().zls_head_mix_gate(_p(acc), _p(talk), _p(v_freq), _p(gate), _i(0 if gate is None else gate.shape[1]), _i(g_col0), batch.ref,
-                                  _i(heads), _i(kv_heads), _i(vdim), _p(out), C.c_int(dt_code(dtype)), _stream()), "head_mix_gate")
+    check(lib().zls_head_mix_gate(_p(acc), _p(ml), _i(n_splits), _p(talk), _p(v_freq), _p(gate), _i(0 if gate is None else gate.shape[1]),
+                                  _i(g_col0), batch.ref, _i(heads), _i(kv_heads), _i(vdim), _p(out), C.c_int(dt_code(dtype)), _stream()),
+          "head_mix_gate")
     return out
 
 
