@@ -86,7 +86,7 @@ __global__ __launch_bounds__(64) void k_moe_route(const float* __restrict__ logi
 
 __global__ __launch_bounds__(1024) void k_moe_align(const int32_t* __restrict__ ids, int n_slots, int top, int n_experts, int tile_m,
                                                     int32_t* __restrict__ sorted_tok, int32_t* __restrict__ slot_pos, int32_t* __restrict__ tiles,
-                                                    int max_tiles) {
+                                                    int max_tiles, int32_t* __restrict__ sorted_exp) {
     extern __shared__ int sh[];
     int* count = sh;                       // [n_experts]
     int* start = sh + n_experts;           // [n_experts + 1]
@@ -132,6 +132,7 @@ __global__ __launch_bounds__(1024) void k_moe_align(const int32_t* __restrict__ 
                 const int pos = at + __popcll(mask & ((1ull << lane) - 1ull));
                 sorted_tok[pos] = i / top;
                 slot_pos[i] = pos;
+                if (sorted_exp) sorted_exp[pos] = e;
             }
             at += __popcll(mask);
         }
@@ -139,6 +140,7 @@ __global__ __launch_bounds__(1024) void k_moe_align(const int32_t* __restrict__ 
     for (int i = tid; i < n_slots; i += 1024) {
         const int e = ids[i];
         if (e < 0 || e >= n_experts) slot_pos[i] = -1;
+        if (sorted_exp && i >= start[n_experts]) sorted_exp[i] = -1;       // sorted positions that no pair takes
     }
 }
 
@@ -179,13 +181,13 @@ extern "C" int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, 
 }
 
 extern "C" int zls_moe_align(const int32_t* ids, int64_t n_slots, int64_t top, int64_t n_experts, int64_t tile_m, int32_t* sorted_tok,
-                             int32_t* slot_pos, int32_t* tiles, int64_t max_tiles, zl_stream_t s) {
+                             int32_t* slot_pos, int32_t* tiles, int64_t max_tiles, int32_t* sorted_exp, zl_stream_t s) {
     ZL_CHECK_ARG(ids && sorted_tok && slot_pos && tiles && n_slots > 0 && top > 0 && n_experts > 0 && tile_m > 0, ZL_EINVAL);
     ZL_CHECK_ARG(n_experts <= 4096 && n_slots < (1 << 30), ZL_ELIMIT);
     ZL_CHECK_ARG(max_tiles >= n_slots / tile_m + n_experts, ZL_ESHAPE);
     const size_t lds = (size_t)(3 * n_experts + 2) * sizeof(int);
     hipLaunchKernelGGL(k_moe_align, dim3(1), dim3(1024), lds, (hipStream_t)s, ids, (int)n_slots, (int)top, (int)n_experts, (int)tile_m, sorted_tok,
-                       slot_pos, tiles, (int)max_tiles);
+                       slot_pos, tiles, (int)max_tiles, sorted_exp);
     return zl_launch_status();
 }
 

@@ -293,6 +293,46 @@ __global__ __launch_bounds__(256) void k_seq_gemv_mfma(const GemmP p) {
         SeqT<ODT>::st(p.y, (size_t)m * p.ldy + col0 + c, red[0][c][m] + red[1][c][m] + red[2][c][m] + red[3][c][m]);
 }
 
+// the grouped product for a FEW rows (decode steps of a mixture of experts): a wave per (sorted row, output column) streams the column's
+// weight row of the row's expert once, 16-byte loads -- a 64-row tile per expert would multiply 63 rows of zeros and leave most of the
+// chip idle.  GATED: the gate row and its up row (16 rows further in the packed block), silu(gate) * up.
+template <int DT, int ODT, bool GATED>
+__global__ __launch_bounds__(256) void k_seq_gemv_grouped(const GemmP p, const int32_t* __restrict__ row_expert, int n_rows) {
+    const int lane = threadIdx.x & 63;
+    const int col = blockIdx.x * 4 + (threadIdx.x >> 6), row = blockIdx.y;
+    const int n_cols = GATED ? p.n / 2 : p.n;
+    if (col >= n_cols || row >= n_rows) return;
+    const int e = row_expert[row];
+    if (e < 0) return;
+    const size_t xr = (size_t)(p.x_rows ? p.x_rows[row] : row) * p.ldx;
+    const size_t w0 = (size_t)e * p.w_stride + (size_t)(GATED ? (col / 16) * 32 + col % 16 : col) * p.k;
+    const size_t w1 = w0 + (size_t)16 * p.k;
+    float a0 = 0.f, a1 = 0.f;
+    if (p.vec && (p.k & 7) == 0) {
+        for (int k = lane * 8; k < p.k; k += 512) {
+            float xv[8], wv[8];
+            Vec8<DT>::ld(p.x, xr + k, xv);
+            Vec8<DT>::ld(p.w, w0 + k, wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a0 = fmaf(wv[i], xv[i], a0);
+            if constexpr (GATED) {
+                Vec8<DT>::ld(p.w, w1 + k, wv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) a1 = fmaf(wv[i], xv[i], a1);
+            }
+        }
+    } else {
+        for (int k = lane; k < p.k; k += 64) {
+            const float xv = SeqT<DT>::ld(p.x, xr + k);
+            a0 = fmaf(SeqT<DT>::ld(p.w, w0 + k), xv, a0);
+            if constexpr (GATED) a1 = fmaf(SeqT<DT>::ld(p.w, w1 + k), xv, a1);
+        }
+    }
+    a0 = zl_wave_sum(a0);
+    if constexpr (GATED) a0 = seq_silu(a0) * zl_wave_sum(a1);
+    if (lane == 0) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, a0);
+}
+
 // 128 x 128 tiles (four times the MFMAs per LDS fragment) when they still fill the chip, 64 x 64 otherwise
 template <int DT, int ODT>
 void launch_tiled(const GemmP& p, hipStream_t hs) {
@@ -372,8 +412,10 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
 // the grouped product of a mixture of experts: one launch over the (expert, row tile) list that zls_moe_align left on the device -- the host
 // never learns how many rows an expert got, the grid covers the upper bound and unused tiles return at once.  64-row tiles.
 extern "C" int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, const int32_t* tiles, int64_t max_tiles,
-                                   void* y, int64_t ldy, int64_t n, int64_t k, int gated, int dtype, int out_dtype, zl_stream_t s) {
+                                   const int32_t* row_expert, int64_t n_rows, void* y, int64_t ldy, int64_t n, int64_t k, int gated, int dtype,
+                                   int out_dtype, zl_stream_t s) {
     ZL_CHECK_ARG(x && w && tiles && y && max_tiles > 0 && n > 0 && k > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(!row_expert || (n_rows > 0 && n_rows <= 65535), ZL_ESHAPE);
     ZL_CHECK_ARG(ldx >= k && n < (1 << 30) && k < (1 << 30) && max_tiles <= 65535, ZL_ESHAPE);
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
     ZL_CHECK_ARG(out_dtype == ZL_F32 || out_dtype == dtype, ZL_EDTYPE);
@@ -385,8 +427,12 @@ extern "C" int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_
     p.vec = (k % unit == 0 && ldx % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
     hipStream_t hs = (hipStream_t)s;
     const dim3 grid((unsigned)((n + 63) / 64), (unsigned)max_tiles);
-#define GROUPED(DT, ODT)                                                                            \
-    if (gated) hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2, true>), grid, dim3(256), 0, hs, p);       \
+    const int64_t n_cols = gated ? n / 2 : n;
+    const dim3 vgrid((unsigned)((n_cols + 3) / 4), (unsigned)(row_expert ? n_rows : 1));
+#define GROUPED(DT, ODT)                                                                                                        \
+    if (row_expert && gated) hipLaunchKernelGGL((k_seq_gemv_grouped<DT, ODT, true>), vgrid, dim3(256), 0, hs, p, row_expert, (int)n_rows);   \
+    else if (row_expert) hipLaunchKernelGGL((k_seq_gemv_grouped<DT, ODT, false>), vgrid, dim3(256), 0, hs, p, row_expert, (int)n_rows);      \
+    else if (gated) hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2, true>), grid, dim3(256), 0, hs, p);                              \
     else hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2, false>), grid, dim3(256), 0, hs, p);
     if (dtype == ZL_BF16) {
         if (out_dtype == ZL_F32) { GROUPED(ZL_BF16, ZL_F32) } else { GROUPED(ZL_BF16, ZL_BF16) }

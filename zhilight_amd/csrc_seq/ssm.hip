@@ -5,7 +5,9 @@
 // k_conv_tail_update  after it: a thread per (sequence, channel) shifts the tail by the portion's length (rows in increasing order, each
 //                     read before it is overwritten)
 // k_ssm_scan          a workgroup per (sequence, head); the state in registers, tokens staged through LDS 16 at a time and walked in order;
-//                     dt, the decay and the state are fp32.
+//                     dt, the decay and the state are fp32.  The same kernel runs linear attention with a scalar decay per head and token
+//                     (zls_decay_scan: x = v, B = k, C = q from columns of one projection, the decay and input scale given per token or
+//                     constant per head, optionally one more value column of ones that carries the normaliser).
 // k_gated_group_norm  y * silu(z), then each of the row's equal parts divided by its own root mean square, times the weight
 #include "seq_common.h"
 
@@ -292,9 +294,12 @@ static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, c
     ZL_CHECK_ARG((int64_t)b->n_seq * n_seg <= 0x7fffffff, ZL_ELIMIT);
     const dim3 grid((unsigned)(b->n_seq * n_seg), (unsigned)heads), block((unsigned)threads);
     hipStream_t hs = (hipStream_t)s;
-    // (up to 256 threads the compiler may use the whole register file for the state and the prefetched chunk)
-#define SCAN(NPT)                                                                                   \
-    if (threads <= 256) hipLaunchKernelGGL((k_ssm_scan<NPT, 256>), grid, block, lds, hs, p, *b);    \
+    // (up to 256 threads the compiler may use the whole register file for the state and the prefetched chunk, up to 512 half of it: the
+    // 32 states, 32 prefetched numbers and 64 offsets of a thread still fit without scratch memory)
+#define SCAN(NPT)                                                                                        \
+    if (threads <= 256) hipLaunchKernelGGL((k_ssm_scan<NPT, 256>), grid, block, lds, hs, p, *b);         \
+    else if (threads <= 512) hipLaunchKernelGGL((k_ssm_scan<NPT, 512>), grid, block, lds, hs, p, *b);    \
+    else if (threads <= 640) hipLaunchKernelGGL((k_ssm_scan<NPT, 640>), grid, block, lds, hs, p, *b);    \
     else hipLaunchKernelGGL((k_ssm_scan<NPT, 1024>), grid, block, lds, hs, p, *b);
 #define SCAN_ANY if (npt <= 8) { SCAN(8) } else if (npt <= 16) { SCAN(16) } else { SCAN(32) }
     if (!segmented) {

@@ -11,7 +11,7 @@
 //                      With all_kv both apply the weights of a query head to the values of EVERY key / value head: mixing the heads'
 //                      weights afterwards is then a small product per token (k_head_mix_gate), sum_g T[h][g] acc[g][c(h)], and no weight
 //                      ever has to wait for another head's normaliser.
-// k_head_mix_gate      a workgroup per token: the splits merged, the mix over heads, the turn back by the token's own position, the gate
+// k_head_mix_gate      a workgroup per (token, kv head): the splits merged, the mix over heads, the turn back by the token's own position, the gate
 // Positions, angles, scores, weights, sums: fp32.  exp / sin / cos are the accurate library versions.
 #include "seq_common.h"
 
@@ -388,49 +388,55 @@ struct MixP {
     void* out;
 };
 
-// a workgroup per token: the splits of every head merged (weights e^(m_s - M) / L into LDS), the mix over heads, the turn back by the
-// token's own position, the gate
+// a workgroup per (token, key / value head c): the splits of every source head merged into LDS (for c's values only), then for the heads of
+// c's group the mix over source heads, the turn back by the token's own position, the gate.  Without a mixing matrix a head's only source
+// is itself.
 template <int DT>
 __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_batch_t b) {
-    extern __shared__ float wsp[];                                        // [heads][n_splits]
-    const int t = blockIdx.x;
+    extern __shared__ float sh[];
+    const int t = blockIdx.x, c = blockIdx.y;
     const int sq = b.tok_seq[t];
     const float pos = (float)(b.seq_pos0[sq] + (t - b.seq_start[sq]));
-    const int per = p.heads / p.kv_heads, half = p.vdim >> 1, S = p.n_splits;
-    const int nv = p.talk ? p.kv_heads * p.vdim : p.vdim;                 // a head's stride in a split of acc
+    const int per = p.heads / p.kv_heads, half = p.vdim >> 1, S = p.n_splits, vd = p.vdim;
+    const int nv = p.talk ? p.kv_heads * vd : vd;                         // a head's stride in a split of acc
+    const int src0 = p.talk ? 0 : c * per, n_src = p.talk ? p.heads : per, col0 = p.talk ? c * vd : 0;
+    float* wsp = sh;                                                      // [n_src][S] weights of the splits
+    float* mg = sh + n_src * S;                                           // [n_src][vd] merged sums
     const float* a = p.acc + (size_t)t * p.heads * S * nv;
-    for (int g = threadIdx.x; g < p.heads; g += 256) {
-        const float* mlp = p.ml + 2 * ((size_t)t * p.heads + g) * S;
+    for (int k = threadIdx.x; k < n_src; k += 256) {
+        const float* mlp = p.ml + 2 * ((size_t)t * p.heads + src0 + k) * S;
         float M = -INFINITY, L = 0.f;
         for (int s = 0; s < S; ++s) M = fmaxf(M, mlp[2 * s]);
-        for (int s = 0; s < S; ++s) L += mlp[2 * s + 1] * expf(mlp[2 * s] - M);
-        for (int s = 0; s < S; ++s) wsp[g * S + s] = mlp[2 * s + 1] > 0.f ? expf(mlp[2 * s] - M) / L : 0.f;
+        for (int s = 0; s < S; ++s) L += mlp[2 * s + 1] > 0.f ? mlp[2 * s + 1] * expf(mlp[2 * s] - M) : 0.f;
+        for (int s = 0; s < S; ++s) wsp[k * S + s] = mlp[2 * s + 1] > 0.f ? expf(mlp[2 * s] - M) / L : 0.f;
     }
     __syncthreads();
-    auto merged = [&](int g, int col) {                                   // head g's sum for column col of its nv
+    for (int e = threadIdx.x; e < n_src * vd; e += 256) {
+        const int k = e / vd, i = e % vd;
+        const float* ak = a + (size_t)(src0 + k) * S * nv + col0 + i;
         float v = 0.f;
         for (int s = 0; s < S; ++s) {
-            const float w = wsp[g * S + s];
-            if (w != 0.f) v = fmaf(w, a[((size_t)g * S + s) * nv + col], v);
+            const float w = wsp[k * S + s];
+            if (w != 0.f) v = fmaf(w, ak[(size_t)s * nv], v);             // (a split without weight may hold anything)
         }
-        return v;
-    };
+        mg[e] = v;
+    }
+    __syncthreads();
     // a thread owns a PAIR (m, m + vdim / 2) of one head (an odd vdim without rotation: the last coordinate alone)
-    const int pairs = p.v_freq ? half : (p.vdim + 1) / 2;
-    for (int w = threadIdx.x; w < p.heads * pairs; w += 256) {
-        const int h = w / pairs, mm = w % pairs;
+    const int pairs = p.v_freq ? half : (vd + 1) / 2;
+    for (int w = threadIdx.x; w < per * pairs; w += 256) {
+        const int h = c * per + w / pairs, mm = w % pairs;
         const int i0 = mm, i1 = mm + pairs;
         float u = 0.f, v = 0.f;
         if (p.talk) {
-            const int c = h / per;
             for (int g = 0; g < p.heads; ++g) {
                 const float tw = p.talk[h * p.heads + g];
-                u = fmaf(tw, merged(g, c * p.vdim + i0), u);
-                if (i1 < p.vdim) v = fmaf(tw, merged(g, c * p.vdim + i1), v);
+                u = fmaf(tw, mg[g * vd + i0], u);
+                if (i1 < vd) v = fmaf(tw, mg[g * vd + i1], v);
             }
         } else {
-            u = merged(h, i0);
-            if (i1 < p.vdim) v = merged(h, i1);
+            u = mg[(h - src0) * vd + i0];
+            if (i1 < vd) v = mg[(h - src0) * vd + i1];
         }
         if (p.v_freq) {
             float sn, cs;
@@ -438,14 +444,14 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
             const float u2 = u * cs + v * sn, v2 = v * cs - u * sn;
             u = u2; v = v2;
         }
-        const size_t o = (size_t)t * p.heads * p.vdim + (size_t)h * p.vdim;
+        const size_t o = (size_t)t * p.heads * vd + (size_t)h * vd;
         if (p.gate) {
-            const float* gr = p.gate + (size_t)t * p.ldg + p.g_col0 + h * p.vdim;
+            const float* gr = p.gate + (size_t)t * p.ldg + p.g_col0 + h * vd;
             u *= seq_sigmoid(gr[i0]);
-            if (i1 < p.vdim) v *= seq_sigmoid(gr[i1]);
+            if (i1 < vd) v *= seq_sigmoid(gr[i1]);
         }
         SeqT<DT>::st(p.out, o + i0, u);
-        if (i1 < p.vdim) SeqT<DT>::st(p.out, o + i1, v);
+        if (i1 < vd) SeqT<DT>::st(p.out, o + i1, v);
     }
 }
 
@@ -521,12 +527,13 @@ extern "C" int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_sp
                                  int dtype, zl_stream_t s) {
     ZL_CHECK_ARG(acc && ml && out && seq_batch_ok(b) && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0 && n_splits >= 1, ZL_EINVAL);
     ZL_CHECK_ARG((!v_freq || vdim % 2 == 0) && (!gate || (g_col0 >= 0 && g_col0 + heads * vdim <= ldg)), ZL_ESHAPE);
-    const size_t lds = (size_t)heads * n_splits * sizeof(float);
-    ZL_CHECK_ARG(lds <= 60 * 1024, ZL_ELIMIT);
+    const int64_t n_src = talk ? heads : heads / kv_heads;
+    const size_t lds = (size_t)n_src * (n_splits + vdim) * sizeof(float);
+    ZL_CHECK_ARG(lds <= 64 * 1024 && kv_heads <= 65535, ZL_ELIMIT);
     MixP p;
     p.acc = acc; p.ml = ml; p.n_splits = (int)n_splits; p.talk = talk; p.v_freq = v_freq; p.gate = gate; p.ldg = ldg; p.g_col0 = (int)g_col0;
     p.heads = (int)heads; p.kv_heads = (int)kv_heads; p.vdim = (int)vdim; p.out = out;
-#define CALL(DT) hipLaunchKernelGGL((k_head_mix_gate<DT>), dim3(b->n_tok), dim3(256), lds, (hipStream_t)s, p, *b);
+#define CALL(DT) hipLaunchKernelGGL((k_head_mix_gate<DT>), dim3(b->n_tok, (unsigned)kv_heads), dim3(256), lds, (hipStream_t)s, p, *b);
     ZLS_DISPATCH(dtype, CALL)
 #undef CALL
     return zl_launch_status();

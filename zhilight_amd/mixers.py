@@ -376,6 +376,7 @@ class RoutedExpertsFF:
         self.width, self.ff, self.experts, self.top, self.identity = width, ff, experts, top, identity
         self.groups, self.keep, self.has_correction, self.renorm = groups, keep, correction, renorm
         self.fused_act = ff % 16 == 0
+        self.few_rows = seqops.MOE_FEW_ROWS
 
     def _pack_gate_up(self, gate, up):
         if not self.fused_act:
@@ -409,11 +410,12 @@ class RoutedExpertsFF:
     def forward(self, h):
         logits = seqops.gemm_nt(h, self.w_router)                                 # fp32 sums of the products
         ids, weights = seqops.moe_route(logits, self.correction, self.groups, self.keep, self.top, self.renorm)
-        sorted_tok, slot_pos, tiles, max_tiles = seqops.moe_align(ids, self.experts)
+        sorted_tok, slot_pos, tiles, max_tiles, sorted_exp = seqops.moe_align(ids, self.experts)
         n_slots = ids.numel()
+        few = sorted_exp if n_slots <= self.few_rows else None                    # decode steps: weight rows streamed per (row, column)
         if self.fused_act:
-            a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype)
+            a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype, row_expert=few)
         else:
-            a = seqops.silu_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots), h.dtype)
-        y = seqops.gemm_nt_grouped(a, None, self.w_down, tiles, max_tiles, n_slots)
+            a = seqops.silu_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, row_expert=few), h.dtype)
+        y = seqops.gemm_nt_grouped(a, None, self.w_down, tiles, max_tiles, n_slots, row_expert=few)
         return seqops.moe_combine(y, slot_pos, ids, weights, h, self.experts)
