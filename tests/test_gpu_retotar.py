@@ -254,6 +254,28 @@ def test_mixing_matrix_crosses_key_value_groups(dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [0, 2])
+def test_attention_without_a_mixing_matrix(dev, dtype, sizes):
+    """the mixer's other form (no tensor `talk`: every head keeps its own weights, and only its own kv head's values are summed) equals the
+    restatement with the identity as mixing matrix"""
+    from zhilight_amd.cache import CacheManager
+    from zhilight_amd.mixers import WindowAttention
+    cfg = O.small_config(("attention",), sizes=sizes)
+    m = cfg["layers"][0]["mixer"]
+    sub = mixer_weights(cfg, 0, 19)
+    sub["talk"] = torch.eye(m["heads"])
+    h = torch.randn(150, cfg["width"], generator=torch.Generator().manual_seed(20)).to(dtype)
+    ref = O.attention_mixer(h.double(), {"x." + k: v for k, v in sub.items()}, "x.", m, EPS)
+    cache = CacheManager(256, 1, dev)
+    mix = WindowAttention("a", cfg["width"], m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"], m["mask"]["size"], m["rot"]["dims"],
+                          m["rot"]["base"], m["rot"]["scaling"]["factor"], EPS, talk=False).load(lambda n: sub[n], "", dtype, dev)
+    mix.bind(cache, dtype)
+    cache.admit("s")
+    (got,) = feed([mix], cache, h, [70, 1, 1, 2, 76], dev)
+    assert mix.talk is None and rel(got, ref) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("portions", [[260], [1, 1, 2, 3, 140, 1, 112], [2] * 20 + [200] + [1] * 20])
 @pytest.mark.parametrize("sizes", [0, 1, 2])
 @pytest.mark.parametrize("segment", [0, 16])

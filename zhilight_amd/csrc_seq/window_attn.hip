@@ -271,21 +271,35 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
     float m_run = -INFINITY, l_run = 0.f;
     const int lo_key = p.window > 0 ? max(0, pos0 - p.window + 1) : 0, hi_key = pos0 + rows - 1;
     int buf = 0;
-    for (int pg = lo_key / 64; pg <= hi_key / 64; ++pg, buf ^= 1) {
+    const int pg_last = hi_key / 64;
+    // the key fragments of a page: A operands straight from the cache rows; the NEXT page's are requested as soon as this page's scores
+    // are issued, and arrive during the softmax and the second product
+    uint4 kf[4][KS];
+    auto load_keys = [&](int pg) {
+        const size_t page = (size_t)pages[pg];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            const uint16_t* kr = kc + ((page * 64 + kb * 16 + nrow) * G + c) * d + 8 * kq;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                kf[kb][ks] = (32 * ks + 8 * kq < d) ? *reinterpret_cast<const uint4*>(kr + 32 * ks) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    load_keys(lo_key / 64);
+    for (int pg = lo_key / 64; pg <= pg_last; ++pg, buf ^= 1) {
         const size_t page = (size_t)pages[pg];
         // ---- scores of the wave's 16 queries against the page's 64 keys
         f4v st[4];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
             st[kb] = (f4v){0.f, 0.f, 0.f, 0.f};
-            const uint16_t* kr = kc + ((page * 64 + kb * 16 + nrow) * G + c) * d + 8 * kq;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const uint4 kf = (32 * ks + 8 * kq < d) ? *reinterpret_cast<const uint4*>(kr + 32 * ks) : make_uint4(0, 0, 0, 0);
-                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, kf), __builtin_bit_cast(b8v, qh[ks]), st[kb], 0, 0, 0);
-                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, kf), __builtin_bit_cast(b8v, ql[ks]), st[kb], 0, 0, 0);
+                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, kf[kb][ks]), __builtin_bit_cast(b8v, qh[ks]), st[kb], 0, 0, 0);
+                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, kf[kb][ks]), __builtin_bit_cast(b8v, ql[ks]), st[kb], 0, 0, 0);
             }
         }
+        if (pg < pg_last) load_keys(pg + 1);
         // st[kb][r]: key pg * 64 + 16 kb + 4 kq + r, query nrow
         float cm = -INFINITY;
         bool vis[4][4];
@@ -300,13 +314,15 @@ __global__ __launch_bounds__(256) void k_window_attention_mfma(const AttnP p, co
         cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
         cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
         const float m_new = fmaxf(m_run, cm);
-        const float corr = m_new == -INFINITY ? 1.0f : expf(m_run - m_new);
+        // (this kernel serves bf16 only: the hardware's exp2 is accurate to 1 ulp of the fp32 result, far inside what the bf16 keys leave)
+        constexpr float kLog2e = 1.4426950408889634f;
+        const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
         float pw[4][4], psum = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                pw[kb][r] = vis[kb][r] ? expf(st[kb][r] - m_new) : 0.f;
+                pw[kb][r] = vis[kb][r] ? __builtin_amdgcn_exp2f((st[kb][r] - m_new) * kLog2e) : 0.f;
                 psum += pw[kb][r];
             }
         psum += __shfl_xor(psum, 16, 64);
