@@ -223,13 +223,13 @@ int zls_moe_route(const float* logits, int64_t n_tok, int64_t n_out, const float
 int zls_moe_align(const int32_t* ids, int64_t n_slots, int64_t top, int64_t n_experts, int64_t tile_m, int32_t* sorted_tok, int32_t* slot_pos,
                   int32_t* tiles, int64_t max_tiles, int32_t* sorted_exp, zl_stream_t s);
 /* y[p] = x[x_rows[p]] . w[expert of p]^T for every sorted position p: w (n_experts, n, k) in `dtype`, x_rows NULL: x[p]; `tiles` from
- * zls_moe_align with tile_m = 64.  gated != 0: n = 2 ff rows per expert, stored as blocks of 16 gate rows followed by their 16 up rows
+ * zls_moe_align with the same tile_m (64 or 128: the workgroup's tile).  gated != 0: n = 2 ff rows per expert, stored as blocks of 16 gate rows followed by their 16 up rows
  * (ff % 16 == 0), and y (.., ff) = silu(gate) * up in out_dtype.  Otherwise y (.., n).
  * row_expert (nullable; sorted_exp of zls_moe_align) with n_rows = the number of sorted positions: the few-rows form -- a wave per (row,
  * output column) streams the weight row once instead of a 64-row tile per expert; the same results up to the order of the fp32 sums. */
 int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, const int32_t* tiles, int64_t max_tiles,
-                        const int32_t* row_expert, int64_t n_rows, void* y, int64_t ldy, int64_t n, int64_t k, int gated, int dtype,
-                        int out_dtype, zl_stream_t s);
+                        int64_t tile_m, const int32_t* row_expert, int64_t n_rows, void* y, int64_t ldy, int64_t n, int64_t k, int gated,
+                        int dtype, int out_dtype, zl_stream_t s);
 /* out[p][c] = silu(gu[p][c]) * gu[p][ff + c]  for rows 0 .. rows - 1 (gu fp32 (rows, 2 ff)), out in `dtype`. */
 int zls_silu_mul(const float* gu, int64_t rows, int64_t ff, void* out, int dtype, zl_stream_t s);
 /* out[t] = sum_k weights[t][k] * (ids[t][k] >= n_experts ? h[t] : y[slot_pos[t * top + k]]), in the order of k; y fp32 (.., width),

@@ -374,6 +374,9 @@ def test_experts_alone(dev, dtype, n_tok, sizes):
     if n_tok <= 5:                                                  # few rows stream weight rows per pair; the tiled kernel gives the same
         ff.few_rows = 0
         assert rel(ff.forward(h.to(dev)), ref) < tol(dtype)
+    if n_tok >= 150:                                                # the 128-row tiles that long shares take
+        ff.tile_m = 128
+        assert rel(ff.forward(h.to(dev)), ref) < tol(dtype)
 
 
 # ------------------------------------------------------------------------------------------------------------------------------------

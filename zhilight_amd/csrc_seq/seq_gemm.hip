@@ -70,8 +70,8 @@ template <> struct Tile<ZL_F32> {
 };
 
 // WT x WT MFMA tiles per wave: the workgroup's output tile is (32 WT) x (32 WT)
-// GATED (WT = 2): the weight rows come in blocks of 16 gate rows followed by their 16 up rows, so that a wave's two column tiles are the gate
-// and the up projection of the same 16 outputs; the epilogue writes silu(gate) * up, half as many columns
+// GATED: the weight rows come in blocks of 16 gate rows followed by their 16 up rows, so that a wave's even column tiles are gates and the
+// odd ones the up projections of the same 16 outputs; the epilogue writes silu(gate) * up, half as many columns
 template <int DT, int ODT, int WT, bool GATED = false>
 __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
     typedef typename Tile<DT>::elem E;
@@ -155,16 +155,20 @@ __global__ __launch_bounds__(256) void k_seq_gemm(const GemmP p) {
         }
     }
     if constexpr (GATED) {
-        static_assert(WT == 2, "the gated epilogue pairs a wave's two column tiles");
-        const int wcol = n0 + wn * 32 + nrow;                   // the gate's weight row; its output column is half the block offset
-        const int col = (n0 + wn * 32) / 2 + nrow;
+        static_assert(WT % 2 == 0, "the gated epilogue pairs a wave's column tiles: even ones are gates, odd ones their up projections");
 #pragma unroll
-        for (int i = 0; i < WT; ++i)
+        for (int jj = 0; jj < WT / 2; ++jj) {
+            const int wcol = n0 + wn * 16 * WT + jj * 32 + nrow;            // the gate's weight row; its output column is half the block offset
+            const int col = (n0 + wn * 16 * WT) / 2 + jj * 16 + nrow;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int row = m0 + wm * 32 + i * 16 + 4 * kq + r;
-                if (row < mlim && wcol < p.n) SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, seq_silu(acc[i][0][r]) * acc[i][1][r]);
-            }
+            for (int i = 0; i < WT; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = m0 + wm * 16 * WT + i * 16 + 4 * kq + r;
+                    if (row < mlim && wcol < p.n)
+                        SeqT<ODT>::st(p.y, (size_t)row * p.ldy + col, seq_silu(acc[i][2 * jj][r]) * acc[i][2 * jj + 1][r]);
+                }
+        }
         return;
     }
 #pragma unroll
@@ -410,11 +414,13 @@ extern "C" int zls_gemm_nt_gather(const void* x, int64_t ldx, const int32_t* x_r
 }
 
 // the grouped product of a mixture of experts: one launch over the (expert, row tile) list that zls_moe_align left on the device -- the host
-// never learns how many rows an expert got, the grid covers the upper bound and unused tiles return at once.  64-row tiles.
+// never learns how many rows an expert got, the grid covers the upper bound and unused tiles return at once.  64- or 128-row tiles (the
+// caller aligns with the same size: 128 when the experts' shares are long enough to fill them).
 extern "C" int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_rows, const void* w, const int32_t* tiles, int64_t max_tiles,
-                                   const int32_t* row_expert, int64_t n_rows, void* y, int64_t ldy, int64_t n, int64_t k, int gated, int dtype,
-                                   int out_dtype, zl_stream_t s) {
+                                   int64_t tile_m, const int32_t* row_expert, int64_t n_rows, void* y, int64_t ldy, int64_t n, int64_t k, int gated,
+                                   int dtype, int out_dtype, zl_stream_t s) {
     ZL_CHECK_ARG(x && w && tiles && y && max_tiles > 0 && n > 0 && k > 0, ZL_EINVAL);
+    ZL_CHECK_ARG(tile_m == 64 || tile_m == 128, ZL_ESHAPE);
     ZL_CHECK_ARG(!row_expert || (n_rows > 0 && n_rows <= 65535), ZL_ESHAPE);
     ZL_CHECK_ARG(ldx >= k && n < (1 << 30) && k < (1 << 30) && max_tiles <= 65535, ZL_ESHAPE);
     ZL_CHECK_ARG(dtype == ZL_BF16 || dtype == ZL_F32, ZL_EDTYPE);
@@ -426,13 +432,15 @@ extern "C" int zls_gemm_nt_grouped(const void* x, int64_t ldx, const int32_t* x_
     const int64_t unit = dtype == ZL_BF16 ? 8 : 4;
     p.vec = (k % unit == 0 && ldx % unit == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0) ? 1 : 0;
     hipStream_t hs = (hipStream_t)s;
-    const dim3 grid((unsigned)((n + 63) / 64), (unsigned)max_tiles);
+    const dim3 grid((unsigned)((n + tile_m - 1) / tile_m), (unsigned)max_tiles);
     const int64_t n_cols = gated ? n / 2 : n;
     const dim3 vgrid((unsigned)((n_cols + 3) / 4), (unsigned)(row_expert ? n_rows : 1));
 #define GROUPED(DT, ODT)                                                                                                        \
     if (row_expert && gated) hipLaunchKernelGGL((k_seq_gemv_grouped<DT, ODT, true>), vgrid, dim3(256), 0, hs, p, row_expert, (int)n_rows);   \
     else if (row_expert) hipLaunchKernelGGL((k_seq_gemv_grouped<DT, ODT, false>), vgrid, dim3(256), 0, hs, p, row_expert, (int)n_rows);      \
+    else if (gated && tile_m == 128) hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 4, true>), grid, dim3(256), 0, hs, p);             \
     else if (gated) hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2, true>), grid, dim3(256), 0, hs, p);                              \
+    else if (tile_m == 128) hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 4, false>), grid, dim3(256), 0, hs, p);                     \
     else hipLaunchKernelGGL((k_seq_gemm<DT, ODT, 2, false>), grid, dim3(256), 0, hs, p);
     if (dtype == ZL_BF16) {
         if (out_dtype == ZL_F32) { GROUPED(ZL_BF16, ZL_F32) } else { GROUPED(ZL_BF16, ZL_BF16) }

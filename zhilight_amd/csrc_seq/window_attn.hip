@@ -431,9 +431,9 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
         const int k = e / vd, i = e % vd;
         const float* ak = a + (size_t)(src0 + k) * S * nv + col0 + i;
         float v = 0.f;
-        for (int s = 0; s < S; ++s) {
-            const float w = wsp[k * S + s];
-            if (w != 0.f) v = fmaf(w, ak[(size_t)s * nv], v);             // (a split without weight may hold anything)
+        for (int s = 0; s < S; ++s) {                                     // (loads first, choice after: they are in flight together)
+            const float w = wsp[k * S + s], x = ak[(size_t)s * nv];
+            v = w != 0.f ? fmaf(w, x, v) : v;                             // (a split without weight may hold anything)
         }
         mg[e] = v;
     }

@@ -377,6 +377,7 @@ class RoutedExpertsFF:
         self.groups, self.keep, self.has_correction, self.renorm = groups, keep, correction, renorm
         self.fused_act = ff % 16 == 0
         self.few_rows = seqops.MOE_FEW_ROWS
+        self.tile_m = None                # rows per expert tile of the grouped products (None: by the experts' average share)
 
     def _pack_gate_up(self, gate, up):
         if not self.fused_act:
@@ -410,12 +411,12 @@ class RoutedExpertsFF:
     def forward(self, h):
         logits = seqops.gemm_nt(h, self.w_router)                                 # fp32 sums of the products
         ids, weights = seqops.moe_route(logits, self.correction, self.groups, self.keep, self.top, self.renorm)
-        sorted_tok, slot_pos, tiles, max_tiles, sorted_exp = seqops.moe_align(ids, self.experts)
+        sorted_tok, slot_pos, tiles, max_tiles, sorted_exp, tm = seqops.moe_align(ids, self.experts, self.tile_m)
         n_slots = ids.numel()
         few = sorted_exp if n_slots <= self.few_rows else None                    # decode steps: weight rows streamed per (row, column)
         if self.fused_act:
-            a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype, row_expert=few)
+            a = seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, gated=True, out_dtype=h.dtype, row_expert=few, tile_m=tm)
         else:
-            a = seqops.silu_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, row_expert=few), h.dtype)
-        y = seqops.gemm_nt_grouped(a, None, self.w_down, tiles, max_tiles, n_slots, row_expert=few)
+            a = seqops.silu_mul(seqops.gemm_nt_grouped(h, sorted_tok, self.w_gu, tiles, max_tiles, n_slots, row_expert=few, tile_m=tm), h.dtype)
+        y = seqops.gemm_nt_grouped(a, None, self.w_down, tiles, max_tiles, n_slots, row_expert=few, tile_m=tm)
         return seqops.moe_combine(y, slot_pos, ids, weights, h, self.experts)

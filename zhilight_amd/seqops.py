@@ -457,7 +457,8 @@ def linear_attn_finish(y, norm_col, q_scale, m_vals, den_eps, heads, vdim, norm_
 
 
 # ---- mixture of experts ------------------------------------------------------------------------------------------------------------------
-MOE_TILE = 64
+MOE_TILE = 64           # rows of an expert's tile in the grouped products; 128 when the average expert gets at least MOE_BIG_SHARE rows
+MOE_BIG_SHARE = 256
 
 
 def moe_route(logits, correction, groups, keep, top, renorm=False):
@@ -476,20 +477,22 @@ def moe_route(logits, correction, groups, keep, top, renorm=False):
 MOE_FEW_ROWS = 64       # up to this many (token, choice) pairs the grouped products stream weight rows per pair instead of tiling
 
 
-def moe_align(ids, n_experts):
-    """(sorted_tok, slot_pos, tiles, max_tiles, sorted_exp) of the (token, choice) pairs sorted by expert"""
+def moe_align(ids, n_experts, tile_m=None):
+    """(sorted_tok, slot_pos, tiles, max_tiles, sorted_exp, tile_m) of the (token, choice) pairs sorted by expert"""
     _cuda(ids)
     n_tok, top = ids.shape
     n_slots = n_tok * top
-    max_tiles = n_slots // MOE_TILE + n_experts
+    if tile_m is None:
+        tile_m = 128 if n_slots >= MOE_BIG_SHARE * n_experts else MOE_TILE
+    max_tiles = n_slots // tile_m + n_experts
     buf = torch.empty(3 * n_slots + 3 * max_tiles, dtype=torch.int32, device=ids.device)
     sorted_tok, slot_pos, sorted_exp, tiles = buf[:n_slots], buf[n_slots:2 * n_slots], buf[2 * n_slots:3 * n_slots], buf[3 * n_slots:]
-    check(lib().zls_moe_align(_p(ids), _i(n_slots), _i(top), _i(n_experts), _i(MOE_TILE), _p(sorted_tok), _p(slot_pos), _p(tiles), _i(max_tiles),
+    check(lib().zls_moe_align(_p(ids), _i(n_slots), _i(top), _i(n_experts), _i(tile_m), _p(sorted_tok), _p(slot_pos), _p(tiles), _i(max_tiles),
                               _p(sorted_exp), _stream()), "moe_align")
-    return sorted_tok, slot_pos, tiles, max_tiles, sorted_exp
+    return sorted_tok, slot_pos, tiles, max_tiles, sorted_exp, tile_m
 
 
-def gemm_nt_grouped(x, x_rows, w, tiles, max_tiles, n_rows, gated=False, out_dtype=torch.float32, row_expert=None):
+def gemm_nt_grouped(x, x_rows, w, tiles, max_tiles, n_rows, gated=False, out_dtype=torch.float32, row_expert=None, tile_m=MOE_TILE):
     """rows of x (gathered by x_rows, or in sorted order) times their expert's block of w (experts, n, k); (n_rows, n or n / 2 gated).
     row_expert (the sorted positions' experts) selects the few-rows kernel."""
     _cuda(x, x_rows, w, tiles, row_expert)
@@ -497,7 +500,7 @@ def gemm_nt_grouped(x, x_rows, w, tiles, max_tiles, n_rows, gated=False, out_dty
     if x.shape[1] != k or x.dtype != w.dtype:
         raise ZLError("gemm_nt_grouped: size K / dtype mismatch")
     out = torch.empty((n_rows, n // 2 if gated else n), dtype=out_dtype, device=x.device)
-    check(lib().zls_gemm_nt_grouped(_p(x), _i(x.stride(0)), _p(x_rows), _p(w), _p(tiles), _i(max_tiles), _p(row_expert), _i(n_rows), _p(out),
+    check(lib().zls_gemm_nt_grouped(_p(x), _i(x.stride(0)), _p(x_rows), _p(w), _p(tiles), _i(max_tiles), _i(tile_m), _p(row_expert), _i(n_rows), _p(out),
                                     _i(out.shape[1]), _i(n), _i(k), C.c_int(int(gated)), C.c_int(dt_code(x.dtype)), C.c_int(dt_code(out_dtype)),
                                     _stream()), "gemm_nt_grouped")
     return out
