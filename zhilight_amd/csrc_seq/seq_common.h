@@ -19,6 +19,15 @@ template <> struct SeqT<ZL_F32> {
 __device__ __forceinline__ float seq_silu(float v) { return v / (1.0f + expf(-v)); }
 __device__ __forceinline__ float seq_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
 __device__ __forceinline__ float seq_softplus(float v) { return v > 20.0f ? v : log1pf(expf(v)); }
+// sine and cosine of an fp32 angle of any size (positions times frequencies reach thousands of radians): the angle is brought into
+// [-pi, pi] in double (exact to 1e-9 for angles up to 2^24), where the fp32 functions take their short path
+__device__ __forceinline__ void seq_sincos(float a, float* sn, float* cs) {
+    const double t = (double)a;
+    const double k = rint(t * 0.15915494309189535);
+    const float r = (float)fma(-k, 6.283185307179586, t);
+    *sn = sinf(r);
+    *cs = cosf(r);
+}
 
 static inline bool seq_batch_ok(const zls_batch_t* b) {
     return b && b->n_seq > 0 && b->n_tok > 0 && b->seq_start && b->seq_pos0 && b->seq_slot && b->tok_seq && b->max_count > 0 &&

@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256) void k_ssm_seg_combine(const ScanP p, const zl
     const int nseg = (whole + p.seg_len - 1) / p.seg_len;
     const int NPs = p.n_state * p.vdim;
     const float* st = p.state + ((size_t)b.seq_slot[sq] * p.heads + h) * NPs;
-    for (int e = threadIdx.x; e < NPs; e += 256) {
+    for (int e = blockIdx.z * 256 + threadIdx.x; e < NPs; e += gridDim.z * 256) {     // (few heads: the state's elements fill the chip instead)
         float S = st[e];
         for (int k = 0; k + 1 < nseg; ++k) {
             const size_t at = ((size_t)sq * p.n_seg + k) * p.heads + h;
@@ -308,7 +308,8 @@ static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, c
     } else {
         p.mode = 1;
         SCAN_ANY
-        hipLaunchKernelGGL(k_ssm_seg_combine, dim3(b->n_seq, (unsigned)heads), dim3(256), 0, hs, p, *b);
+        const int64_t want_z = (1024 + b->n_seq * heads - 1) / (b->n_seq * heads), have_z = (n_state * vdim + 255) / 256;
+        hipLaunchKernelGGL(k_ssm_seg_combine, dim3(b->n_seq, (unsigned)heads, (unsigned)(want_z < have_z ? want_z : have_z)), dim3(256), 0, hs, p, *b);
         p.mode = 2;
         SCAN_ANY
     }

@@ -12,7 +12,8 @@
 //                      weights afterwards is then a small product per token (k_head_mix_gate), sum_g T[h][g] acc[g][c(h)], and no weight
 //                      ever has to wait for another head's normaliser.
 // k_head_mix_gate      a workgroup per (token, kv head): the splits merged, the mix over heads, the turn back by the token's own position, the gate
-// Positions, angles, scores, weights, sums: fp32.  exp / sin / cos are the accurate library versions.
+// Positions, angles, scores, weights, sums: fp32.  exp is the accurate library version (the bf16 matrix-core kernel: the hardware's exp2);
+// sin / cos take an angle reduced in double (seq_sincos).
 #include "seq_common.h"
 
 namespace {
@@ -37,7 +38,7 @@ __device__ __forceinline__ void rope_head(float* v, const float* src, int size, 
                 const bool lo = i < half;
                 const float other = src[lo ? i + half : i - half];
                 float sn, cs;
-                sincosf(pos * freq[lo ? i : i - half], &sn, &cs);
+                seq_sincos(pos * freq[lo ? i : i - half], &sn, &cs);
                 o = lo ? o * cs - other * sn : o * cs + other * sn;
             }
             ss = fmaf(o, o, ss);
@@ -431,6 +432,7 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
         const int k = e / vd, i = e % vd;
         const float* ak = a + (size_t)(src0 + k) * S * nv + col0 + i;
         float v = 0.f;
+#pragma unroll 4
         for (int s = 0; s < S; ++s) {                                     // (loads first, choice after: they are in flight together)
             const float w = wsp[k * S + s], x = ak[(size_t)s * nv];
             v = w != 0.f ? fmaf(w, x, v) : v;                             // (a split without weight may hold anything)
@@ -456,7 +458,7 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
         }
         if (p.v_freq) {
             float sn, cs;
-            sincosf(pos * p.v_freq[mm], &sn, &cs);                        // turned by -pos: (u cs + v sn, v cs - u sn)
+            seq_sincos(pos * p.v_freq[mm], &sn, &cs);                        // turned by -pos: (u cs + v sn, v cs - u sn)
             const float u2 = u * cs + v * sn, v2 = v * cs - u * sn;
             u = u2; v = v2;
         }
