@@ -419,14 +419,21 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
     const int src0 = p.talk ? 0 : c * per, n_src = p.talk ? p.heads : per, col0 = p.talk ? c * vd : 0;
     float* wsp = sh;                                                      // [n_src][S] weights of the splits
     float* mg = sh + n_src * S;                                           // [n_src][vd] merged sums
+    float* tk = mg + n_src * vd;                                          // [per][heads] this group's rows of the mixing matrix
     const float* a = p.acc + (size_t)t * p.heads * S * nv;
-    for (int k = threadIdx.x; k < n_src; k += 256) {
-        const float* mlp = p.ml + 2 * ((size_t)t * p.heads + src0 + k) * S;
-        float M = -INFINITY, L = 0.f;
-        for (int s = 0; s < S; ++s) M = fmaxf(M, mlp[2 * s]);
-        for (int s = 0; s < S; ++s) L += mlp[2 * s + 1] > 0.f ? mlp[2 * s + 1] * expf(mlp[2 * s] - M) : 0.f;
-        for (int s = 0; s < S; ++s) wsp[k * S + s] = mlp[2 * s + 1] > 0.f ? expf(mlp[2 * s] - M) / L : 0.f;
+    const int lane = threadIdx.x & 63;
+    for (int k = threadIdx.x >> 6; k < n_src; k += 4) {                   // a wave per source head, a lane per split: all loads at once
+        const float2* mlp = reinterpret_cast<const float2*>(p.ml) + ((size_t)t * p.heads + src0 + k) * S;
+        float M = -INFINITY;
+        for (int s = lane; s < S; s += 64) M = fmaxf(M, mlp[s].x);
+        M = zl_wave_max(M);
+        float L = 0.f;
+        for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; L += v.y > 0.f ? v.y * expf(v.x - M) : 0.f; }
+        L = zl_wave_sum(L);
+        for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; wsp[k * S + s] = v.y > 0.f ? expf(v.x - M) / L : 0.f; }
     }
+    if (p.talk)
+        for (int i = threadIdx.x; i < per * p.heads; i += 256) tk[i] = p.talk[(size_t)c * per * p.heads + i];
     __syncthreads();
     for (int e = threadIdx.x; e < n_src * vd; e += 256) {
         const int k = e / vd, i = e % vd;
@@ -448,7 +455,7 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
         float u = 0.f, v = 0.f;
         if (p.talk) {
             for (int g = 0; g < p.heads; ++g) {
-                const float tw = p.talk[h * p.heads + g];
+                const float tw = tk[(h - c * per) * p.heads + g];
                 u = fmaf(tw, mg[g * vd + i0], u);
                 if (i1 < vd) v = fmaf(tw, mg[g * vd + i1], v);
             }
@@ -546,7 +553,7 @@ extern "C" int zls_head_mix_gate(const float* acc, const float* ml, int64_t n_sp
     ZL_CHECK_ARG(acc && ml && out && seq_batch_ok(b) && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0 && n_splits >= 1, ZL_EINVAL);
     ZL_CHECK_ARG((!v_freq || vdim % 2 == 0) && (!gate || (g_col0 >= 0 && g_col0 + heads * vdim <= ldg)), ZL_ESHAPE);
     const int64_t n_src = talk ? heads : heads / kv_heads;
-    const size_t lds = (size_t)n_src * (n_splits + vdim) * sizeof(float);
+    const size_t lds = (size_t)(n_src * (n_splits + vdim) + (talk ? heads / kv_heads * heads : 0)) * sizeof(float);
     ZL_CHECK_ARG(lds <= 64 * 1024 && kv_heads <= 65535, ZL_ELIMIT);
     MixP p;
     p.acc = acc; p.ml = ml; p.n_splits = (int)n_splits; p.talk = talk; p.v_freq = v_freq; p.gate = gate; p.ldg = ldg; p.g_col0 = (int)g_col0;
