@@ -422,29 +422,52 @@ __global__ __launch_bounds__(256) void k_head_mix_gate(const MixP p, const zls_b
     float* tk = mg + n_src * vd;                                          // [per][heads] this group's rows of the mixing matrix
     const float* a = p.acc + (size_t)t * p.heads * S * nv;
     const int lane = threadIdx.x & 63;
-    for (int k = threadIdx.x >> 6; k < n_src; k += 4) {                   // a wave per source head, a lane per split: all loads at once
-        const float2* mlp = reinterpret_cast<const float2*>(p.ml) + ((size_t)t * p.heads + src0 + k) * S;
-        float M = -INFINITY;
-        for (int s = lane; s < S; s += 64) M = fmaxf(M, mlp[s].x);
-        M = zl_wave_max(M);
-        float L = 0.f;
-        for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; L += v.y > 0.f ? v.y * expf(v.x - M) : 0.f; }
-        L = zl_wave_sum(L);
-        for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; wsp[k * S + s] = v.y > 0.f ? expf(v.x - M) / L : 0.f; }
-    }
+    if (S > 1)
+        for (int k = threadIdx.x >> 6; k < n_src; k += 4) {               // a wave per source head, a lane per split: all loads at once
+            const float2* mlp = reinterpret_cast<const float2*>(p.ml) + ((size_t)t * p.heads + src0 + k) * S;
+            float M = -INFINITY;
+            for (int s = lane; s < S; s += 64) M = fmaxf(M, mlp[s].x);
+            M = zl_wave_max(M);
+            float L = 0.f;
+            for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; L += v.y > 0.f ? v.y * expf(v.x - M) : 0.f; }
+            L = zl_wave_sum(L);
+            for (int s = lane; s < S; s += 64) { const float2 v = mlp[s]; wsp[k * S + s] = v.y > 0.f ? expf(v.x - M) / L : 0.f; }
+        }
     if (p.talk)
         for (int i = threadIdx.x; i < per * p.heads; i += 256) tk[i] = p.talk[(size_t)c * per * p.heads + i];
     __syncthreads();
-    for (int e = threadIdx.x; e < n_src * vd; e += 256) {
-        const int k = e / vd, i = e % vd;
-        const float* ak = a + (size_t)(src0 + k) * S * nv + col0 + i;
-        float v = 0.f;
-#pragma unroll 4
-        for (int s = 0; s < S; ++s) {                                     // (loads first, choice after: they are in flight together)
-            const float w = wsp[k * S + s], x = ak[(size_t)s * nv];
-            v = w != 0.f ? fmaf(w, x, v) : v;                             // (a split without weight may hold anything)
+    // merged sums: 8 elements per thread at a time, their loads of one split in flight together
+    for (int e0 = 0; e0 < n_src * vd; e0 += 8 * 256) {
+        float v[8];
+        const float* src[8];
+        int kk[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int e = min(e0 + 256 * r + (int)threadIdx.x, n_src * vd - 1);
+            kk[r] = e / vd;
+            src[r] = a + (size_t)(src0 + kk[r]) * S * nv + col0 + e % vd;
+            v[r] = 0.f;
         }
-        mg[e] = v;
+        if (S == 1) {                                                     // one split: its own weight sum normalises it
+#pragma unroll
+            for (int r = 0; r < 8; ++r) v[r] = (1.0f / p.ml[2 * ((size_t)t * p.heads + src0 + kk[r]) + 1]) * *src[r];
+        } else {
+            for (int s = 0; s < S; ++s) {
+                float x[8];
+#pragma unroll
+                for (int r = 0; r < 8; ++r) x[r] = src[r][(size_t)s * nv];
+#pragma unroll
+                for (int r = 0; r < 8; ++r) {
+                    const float w = wsp[kk[r] * S + s];
+                    v[r] = w != 0.f ? fmaf(w, x[r], v[r]) : v[r];         // (a split without weight may hold anything)
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int e = e0 + 256 * r + (int)threadIdx.x;
+            if (e < n_src * vd) mg[e] = v[r];
+        }
     }
     __syncthreads();
     // a thread owns a PAIR (m, m + vdim / 2) of one head (an odd vdim without rotation: the last coordinate alone)
