@@ -386,6 +386,7 @@ CONFIGS = {
     "all_kinds": dict(order=("lightning", "mlstm", "attention", "shared")),
     "attention_first": dict(order=("attention", "mlstm", "shared", "lightning", "shared"), width=100, sizes=1, no_mlp_at=(1, 4)),
     "wide_heads": dict(order=("mlstm", "attention", "lightning"), width=90, vocab=131, sizes=2, no_mlp_at=(0,)),
+    "two_lenders": dict(order=("attention", "shared", "lightning", "attention", "shared", "mlstm"), width=64, vocab=50, sizes=3, no_mlp_at=(2,)),
 }
 
 
