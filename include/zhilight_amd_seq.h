@@ -112,7 +112,8 @@ int zls_conv_tail_update(const float* proj, int64_t ld, int64_t col0, float* tai
  *   dt = softplus(dt_raw + dt_bias_h);  S <- exp(-exp(a_log_h) dt) S + dt B x^T;  y = S^T C + d_h x
  * xbc fp32 (n_tok, heads * vdim + 2 groups * n_state) = [x | B | C] after the convolution; dt_raw = proj[t][dt_col0 + h] (fp32, ld);
  * state fp32 (slots, heads, n_state, vdim), read at the start and written back at the end; y fp32 (n_tok, heads * vdim).
- * Head h uses group h / (heads / groups).  vdim * ceil_pow2(n_state / 32) <= 1024. */
+ * Head h uses group h / (heads / groups).  A workgroup holds up to 1024 / ceil_pow2(n_state / 32) value columns of a head; wider heads
+ * are cut into column parts (columns never meet in the recurrence).  vdim <= 1024, n_state <= 2048. */
 int zls_ssm_scan(const float* xbc, const float* proj, int64_t ld, int64_t dt_col0, const float* dt_bias, const float* a_log, const float* d,
                  float* state, int64_t heads, int64_t vdim, int64_t n_state, int64_t groups, const zls_batch_t* b, float* y, void* workspace,
                  int64_t seg_len, zl_stream_t s);

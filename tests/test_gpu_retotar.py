@@ -326,6 +326,30 @@ def test_mlstm_alone(dev, dtype, portions, sizes, gates):
     assert float(mix.state[0].abs().max()) == 0.0 and float(mix.m_state[0].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("kind", ["lightning", "mlstm"])
+def test_recurrent_heads_wider_than_one_workgroup(dev, kind):
+    """value sizes whose columns (times the lanes that share a column's states) exceed a workgroup: the scan cuts the head into column parts"""
+    from zhilight_amd.cache import CacheManager
+    from zhilight_amd.mixers import DecayLinearAttention, MLSTMMixer
+    cfg = O.small_config((kind,), sizes=2)
+    m = cfg["layers"][0]["mixer"]
+    m.update(dict(heads=1, dim=100, vdim=300, decay=[0.98]) if kind == "lightning" else dict(heads=2, dim=72, vdim=260))
+    sub = mixer_weights(cfg, 0, 23)
+    h = torch.randn(90, cfg["width"], generator=torch.Generator().manual_seed(24))
+    sd = {"x." + k: v for k, v in sub.items()}
+    ref = (O.lightning_mixer if kind == "lightning" else O.mlstm_mixer)(h.double(), sd, "x.", m, EPS)
+    cache = CacheManager(128, 1, dev)
+    if kind == "lightning":
+        mix = DecayLinearAttention("l", cfg["width"], m["heads"], m["dim"], m["vdim"], m["decay"], EPS)
+    else:
+        mix = MLSTMMixer("m", cfg["width"], m["heads"], m["dim"], m["vdim"], m["gate_cap"], EPS)
+    mix.load(lambda n: sub[n], "", torch.float32, dev).bind(cache, torch.float32)
+    mix.scan_segment = 16
+    cache.admit("s")
+    (got,) = feed([mix], cache, h, [1, 2, 50, 1, 36], dev)
+    assert rel(got, ref) < F32_TOL
+
+
 def build_experts(cfg, sub, dtype, dev):
     from zhilight_amd.mixers import RoutedExpertsFF
     f = cfg["layers"][0]["mlp"]

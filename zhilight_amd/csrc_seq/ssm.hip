@@ -60,6 +60,7 @@ struct ScanP {
     // `proj` (x = v, B = k, C = q, each head its own), through SiLU when act is set; the input scale is gain_t[t][h] (or 1), the decay
     // decay_t[t][h] (or the constant decay_h[h]); with `ones` the last of the vdim columns is not loaded but 1 for every token
     int kind, act, ones, q_col0, k_col0, v_col0;
+    int cols;                                                // value columns per workgroup (all of them, or a part: blockIdx.z picks it)
     const float* decay_h; const float* decay_t; const float* gain_t;
 };
 
@@ -81,8 +82,10 @@ __global__ __launch_bounds__(MAXT) void k_ssm_scan(const ScanP p, const zls_batc
     float* dts = lds + CH * WL;                    // [CH] dt | [CH] decay
     for (int i = threadIdx.x; i < CH * WL; i += blockDim.x) rows[i] = 0.f;
     const int sq = blockIdx.x / p.n_seg, seg = blockIdx.x % p.n_seg, h = blockIdx.y, tid = threadIdx.x, nthr = blockDim.x;
-    const int pp = tid / p.ngl, g = tid % p.ngl;
-    const bool active = pp < P;
+    // (columns never meet in the recurrence: wide heads are cut into column parts, each workgroup stages the whole token row and keeps
+    // the states of its own columns)
+    const int pp = blockIdx.z * p.cols + tid / p.ngl, g = tid % p.ngl;
+    const bool active = tid / p.ngl < p.cols && pp < P;
     const bool lin = p.kind == 1;
     const int grp = lin ? 0 : h / (p.heads / p.groups);
     const int inner = p.heads * P, chan = lin ? (int)p.ld : inner + 2 * p.groups * N;
@@ -269,16 +272,20 @@ static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, c
     // ngl lanes share a column: the smallest power of two that leaves a thread at most 32 states
     int64_t ngl = 1;
     while ((n_state + ngl - 1) / ngl > 32) ngl <<= 1;
-    ZL_CHECK_ARG(ngl <= 64 && ngl * vdim <= 1024, ZL_ELIMIT);
+    ZL_CHECK_ARG(ngl <= 64, ZL_ELIMIT);
+    const int64_t cols = ngl * vdim <= 1024 ? vdim : 1024 / ngl, col_parts = (vdim + cols - 1) / cols;
+    p.cols = (int)cols;
     const int64_t npt = ((n_state + ngl - 1) / ngl + 3) / 4 * 4;
-    const int64_t threads = (ngl * vdim + 63) / 64 * 64;
+    const int64_t threads = (ngl * cols + 63) / 64 * 64;
     p.heads = (int)heads; p.vdim = (int)vdim; p.n_state = (int)n_state;
     p.ngl = (int)ngl; p.npt = (int)npt;
     const int64_t row = vdim + 2 * n_state;
-    const int64_t kp = (row + threads - 1) / threads;                  // register slots a staged token row takes per thread
+    int64_t kp = (row + threads - 1) / threads;                        // register slots a staged token row takes per thread
+    const size_t row_bytes = (size_t)((vdim + 3) / 4 * 4 + 2 * ngl * (npt + 4) + 2) * sizeof(float);
+    while (kp < kScanSlots && (kScanSlots / kp) * row_bytes > 64 * 1024) ++kp;      // long rows: fewer tokens staged at a time
     ZL_CHECK_ARG(kp <= kScanSlots, ZL_ELIMIT);
     p.kp = (int)kp;
-    const size_t lds = (size_t)(kScanSlots / kp) * ((vdim + 3) / 4 * 4 + 2 * ngl * (npt + 4) + 2) * sizeof(float);
+    const size_t lds = (kScanSlots / kp) * row_bytes;
     ZL_CHECK_ARG(lds <= 64 * 1024, ZL_ELIMIT);
     // portions longer than seg_len (with a workspace): every segment from a zero state in parallel, the segments' start states by a short
     // serial pass over their end states, then every segment again from its true start state -- twice the arithmetic, 1 / segments of the
@@ -292,7 +299,7 @@ static int launch_scan(ScanP& p, int64_t heads, int64_t vdim, int64_t n_state, c
     p.seg_init = p.seg_state + per * n_state * vdim;
     p.seg_prod = p.seg_init + per * n_state * vdim;
     ZL_CHECK_ARG((int64_t)b->n_seq * n_seg <= 0x7fffffff, ZL_ELIMIT);
-    const dim3 grid((unsigned)(b->n_seq * n_seg), (unsigned)heads), block((unsigned)threads);
+    const dim3 grid((unsigned)(b->n_seq * n_seg), (unsigned)heads, (unsigned)col_parts), block((unsigned)threads);
     hipStream_t hs = (hipStream_t)s;
     // (up to 256 threads the compiler may use the whole register file for the state and the prefetched chunk, up to 512 half of it: the
     // 32 states, 32 prefetched numbers and 64 offsets of a thread still fit without scratch memory)
