@@ -1,4 +1,4 @@
-"""Plain, slow restatement of the Retotar design in float64 on the CPU: what the product path (zhilight_amd/retotar.py, mixers.py, moe.py,
+"""Plain, slow restatement of the Retotar design in float64 on the CPU: what the product path (zhilight_amd/retotar.py, mixers.py,
 engine.py and the kernels of csrc_seq/) is held against.  One function per mechanism, whole sequences only, no cache, no batching,
 nothing shared with the product code.  Weights are a dict name -> torch tensor with the checkpoint's own tensor names; `m` is a layer's
 "mixer" entry of the configuration, `f` its "mlp" entry.
